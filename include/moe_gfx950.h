@@ -51,8 +51,9 @@ int moe_abi_version(void);
 
 /* ---- routing ------------------------------------------------------------------------
  * Replaces `torch.topk(gate_logits, k)` + `F.softmax(weights)` (mlp.py:101-103).
- * logits [T,E] (bf16 or f32); optional bias f32 [E] added in fp32 before selection (NULL
- * for the reference behaviour).  Ties: the lower expert index wins; slots are in
+ * logits [T,E] (bf16 or f32); optional bias f32 [E] added to the logits in fp32 (NULL for the
+ * reference behaviour): selection AND the softmax over the selected values use logit + bias.
+ * Ties: the lower expert index wins; slots are in
  * descending-logit order.  ids_out int32 [T*k], gates_out f32 [T*k]. */
 int moe_router_topk_fwd(const void* logits, int logits_dtype, const float* bias, int64_t T,
                         int64_t E, int64_t k, int32_t* ids_out, float* gates_out,
@@ -74,6 +75,16 @@ int64_t moe_dispatch_workspace_bytes(int64_t R, int64_t E);
 int moe_histogram_scan(const int32_t* ids, int64_t R, int64_t E, int32_t* counts,
                        int32_t* offs, int32_t* pos_to_row, int32_t* row_to_pos,
                        void* workspace, int64_t workspace_bytes, void* stream);
+/* The same, and *bad_ids (device int32, may be NULL) receives the number of ids outside [0,E).
+ * Such a row is counted and placed with the nearest valid expert (0 or E-1), so that the
+ * permutation stays a bijection and no kernel downstream reads out of bounds; a caller that
+ * takes ids from outside (mlp.py:122, `received_experts` after the all-to-all) reads the count
+ * when it next synchronises anyway and rejects the step if it is not zero.  (The reference's
+ * bincount/argsort would raise or misplace silently on such ids.) */
+int moe_histogram_scan_checked(const int32_t* ids, int64_t R, int64_t E, int32_t* counts,
+                               int32_t* offs, int32_t* pos_to_row, int32_t* row_to_pos,
+                               int32_t* bad_ids, void* workspace, int64_t workspace_bytes,
+                               void* stream);
 
 /* Replaces `repeat_interleave(k)` + the two row gathers (mlp.py:104, 108, 124):
  * xp[pos,:] = bf16(x[pos_to_row[pos] / k, :]).  x [T,H] (x_dtype), xp bf16 [R,H]. */

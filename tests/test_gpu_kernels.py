@@ -130,6 +130,43 @@ def test_histogram_scan_bit_exact(ops, case):
     assert np.array_equal(r2p.cpu().numpy(), or2p.astype(np.int32))
 
 
+def test_histogram_scan_counts_ids_out_of_range(pkg, ops):
+    """Expert ids outside [0, E): counted on the device, rows placed with the nearest valid
+    expert (the result equals the sort of the clipped ids), nothing read or written out of
+    bounds; valid inputs report zero.  `experts_rows(check_ids=True)` turns the count into an
+    exception."""
+    _say("histogram_scan with invalid ids")
+    rng = np.random.default_rng(11)
+    E, R = 12, 3000
+    ids = rng.integers(0, E, size=R)
+    where = rng.choice(R, size=37, replace=False)
+    ids[where[:20]] = rng.integers(E, E + 1000, size=20)
+    ids[where[20:]] = -rng.integers(1, 1000, size=17)
+    d = torch.from_numpy(ids.astype(np.int32)).cuda()
+    counts, offs, p2r, r2p, bad = ops.histogram_scan(d, E, return_bad=True)
+    assert bad.item() == 37
+    clipped = np.clip(ids, 0, E - 1)
+    oc, ostarts = O.counts_offsets(clipped, E)
+    op2r, or2p = O.stable_permutation(clipped)
+    assert np.array_equal(counts.cpu().numpy(), oc.astype(np.int32))
+    assert np.array_equal(offs.cpu().numpy(), ostarts)
+    assert np.array_equal(p2r.cpu().numpy(), op2r.astype(np.int32))
+    assert np.array_equal(r2p.cpu().numpy(), or2p.astype(np.int32))
+    good = torch.from_numpy(clipped.astype(np.int32)).cuda()
+    assert ops.histogram_scan(good, E, return_bad=True)[4].item() == 0
+    assert ops.histogram_scan(good[:0], E, return_bad=True)[4].item() == 0
+    H, I = 64, 32
+    g = torch.Generator().manual_seed(3)
+    rows = torch.randn(R, H, generator=g).to(torch.bfloat16).cuda()
+    ws = [(torch.randn(*s_, generator=g) * 0.1).to(torch.bfloat16).cuda() for s_ in ((E, I, H), (E, I, H), (E, H, I))]
+    out, rt = pkg.experts_rows(rows, good, *ws, return_routing=True, check_ids=True)
+    assert rt["bad_ids"].item() == 0
+    with pytest.raises(ValueError, match="37 of 3000"):
+        pkg.experts_rows(rows, d, *ws, check_ids=True)
+    out_bad, rt = pkg.experts_rows(rows, d, *ws, return_routing=True)   # unchecked: runs, and says so
+    assert rt["bad_ids"].item() == 37 and torch.equal(out_bad, out)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("T,H,k,E", [(300, 256, 2, 8), (64, 2048, 8, 64), (5, 8, 1, 3), (33, 1032, 3, 5),
                                      (17, 4096, 2, 4)])

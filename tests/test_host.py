@@ -35,7 +35,7 @@ def test_library_exports_every_declared_symbol():
     assert sorted(names) == sorted(pkg.lib.SIGNATURES)
     L = pkg.lib.load()
     assert L.abi_version == 100
-    assert L.cdll.moe_dispatch_workspace_bytes(1000, 8) == 4 * 8 * 4
+    assert L.cdll.moe_dispatch_workspace_bytes(1000, 8) == 4 * (8 + 1) * 4
 
 
 def test_module_constructor_contract_cpu():

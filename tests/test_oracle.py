@@ -268,6 +268,123 @@ def test_rows_entry_forward_backward():
     assert not b["dw1"][2].any()
 
 
+# ----------------------------------------------------------------------------- bf16 storage emulation
+def _rb(t):
+    return t.to(torch.bfloat16).to(t.dtype)
+
+
+class _RoundValue(torch.autograd.Function):
+    """bf16 rounding of the value; the gradient passes unchanged."""
+    @staticmethod
+    def forward(ctx, t):
+        return _rb(t)
+
+    @staticmethod
+    def backward(ctx, gr):
+        return gr
+
+
+class _RoundGrad(torch.autograd.Function):
+    """The value passes unchanged; the gradient is rounded to bf16."""
+    @staticmethod
+    def forward(ctx, t):
+        return t.view_as(t)
+
+    @staticmethod
+    def backward(ctx, gr):
+        return _rb(gr)
+
+
+class _StoredSwiGLU(torch.autograd.Function):
+    """act = bf16(silu(g) * u) from unrounded g, u; backward differentiates silu(g)*u with the
+    library's autograd AT the bf16-stored g, u and rounds both results to bf16."""
+    @staticmethod
+    def forward(ctx, g, u):
+        ctx.save_for_backward(_rb(g), _rb(u))
+        return _rb(F.silu(g) * u)
+
+    @staticmethod
+    def backward(ctx, dact):
+        gs, us = (t.detach().requires_grad_(True) for t in ctx.saved_tensors)
+        with torch.enable_grad():
+            a = F.silu(gs) * us
+        dg, du = torch.autograd.grad(a, (gs, us), dact)
+        return _rb(dg), _rb(du)
+
+
+@pytest.mark.parametrize("T,H,E,I,k", [(96, 64, 6, 48, 2), (40, 32, 4, 24, 3), (64, 48, 5, 40, 1)])
+def test_bf16_emulation_matches_an_autograd_restatement_with_the_same_rounding_points(T, H, E, I, k):
+    """The oracle's `emulate_bf16` mode (the yardstick of the GPU tolerance rule) against an
+    independent restatement: the reference's padded-bmm formulation (mlp.py:133-167) under the
+    library's autograd, with bf16 rounding inserted as autograd nodes at the points where the
+    device stores bf16 (g, u, act, y forward; gate*dy, dg, du, d rows, dlogits backward).  Values
+    that do not depend on how the gate gradient is formed must agree to fp32 summation order; the
+    gate gradient itself is <dy, y> here and <dact, act>/gate there (equal in exact arithmetic),
+    so it and what follows from it agree to bf16 rounding."""
+    x, wr, w1, w3, w2 = (_rb(t) for t in _mk(T, H, E, I, seed=70 + T, std=0.2))
+    dy = _rb(torch.randn(T, H, generator=torch.Generator().manual_seed(5)))
+    logits = _rb(F.linear(x, wr))
+    fe = O.moe_forward(x, wr, w1, w3, w2, k, logits=logits, emulate_bf16=True)
+    be = O.moe_backward(fe, dy, wr, w1, w3, w2, emulate_bf16=True)
+
+    ids = torch.from_numpy(fe["ids"])
+    lx, lw1, lw3, lw2 = (t.clone().requires_grad_(True) for t in (x, w1, w3, w2))
+    llog = logits.clone().requires_grad_(True)
+    weights = F.softmax(torch.gather(llog, 1, ids).float(), dim=-1).view(-1)
+    selected = ids.view(-1)
+    flat_x = lx.repeat_interleave(k, dim=0)
+    sort_idx = torch.argsort(selected, stable=True)
+    local_x = _RoundGrad.apply(flat_x[sort_idx])
+    local_e = selected[sort_idx]
+    counts = torch.bincount(local_e, minlength=E)
+    starts = torch.cumsum(counts, 0) - counts
+    rel = torch.arange(T * k) - starts[local_e]
+    padded = torch.zeros(E, int(counts.max()), H).index_put((local_e, rel), local_x)
+    act = _StoredSwiGLU.apply(torch.bmm(padded, lw1.transpose(1, 2)), torch.bmm(padded, lw3.transpose(1, 2)))
+    down = _RoundGrad.apply(_RoundValue.apply(torch.bmm(act, lw2.transpose(1, 2))[local_e, rel]))
+    out = (down[torch.argsort(sort_idx)] * weights.unsqueeze(-1)).view(T, k, H).sum(1)
+    assert torch.allclose(out, fe["out"], rtol=1e-5, atol=1e-6)
+    out.backward(dy)
+
+    tight = dict(rtol=2e-5, atol=2e-6)
+    assert torch.allclose(lw1.grad, be["dw1"], **tight)
+    assert torch.allclose(lw3.grad, be["dw3"], **tight)
+    assert torch.allclose(lw2.grad, be["dw2"], **tight)
+    assert torch.allclose(lx.grad, be["dx_expert"], **tight)   # router path not in this graph's x
+    # gate-gradient side: two estimators of the same number, a bf16 rounding apart
+    dl = llog.grad
+    scale = be["dlogits"].abs().max().item()
+    assert (dl - be["dlogits"]).abs().max().item() <= 2e-2 * scale
+    dl_r = _rb(dl)
+    assert ((dl_r.t() @ x) - be["dwr"]).norm() <= 2e-2 * be["dwr"].norm()
+    assert ((dl_r @ wr) - be["dx_router"]).norm() <= 2e-2 * be["dx_router"].norm()
+    # and the emulation differs from the unrounded oracle (it is not a no-op) by bf16-sized amounts
+    f = O.moe_forward(x, wr, w1, w3, w2, k, logits=logits)
+    b = O.moe_backward(f, dy, wr, w1, w3, w2)
+    for n in ("dw1", "dw3", "dw2"):
+        rel_err = ((be[n] - b[n]).norm() / b[n].norm()).item()
+        assert 1e-5 < rel_err < 1e-2, (n, rel_err)
+
+
+def test_bf16_emulation_of_the_rows_entry_matches_the_layer_emulation():
+    """`experts_rows_*` with `emulate_bf16` is the k = 1, gate = 1 case of the layer's emulation
+    (pinned above): same dyp, dg, du, d rows and weight gradients."""
+    T, H, E, I = 80, 32, 5, 24
+    x, wr, w1, w3, w2 = (_rb(t) for t in _mk(T, H, E, I, seed=90, std=0.2))
+    dy = _rb(torch.randn(T, H, generator=torch.Generator().manual_seed(6)))
+    logits = _rb(F.linear(x, wr))
+    fe = O.moe_forward(x, wr, w1, w3, w2, 1, logits=logits, emulate_bf16=True)
+    be = O.moe_backward(fe, dy, wr, w1, w3, w2, emulate_bf16=True)
+    assert torch.equal(fe["gates"], torch.ones(T, 1))
+    ids = fe["ids"].reshape(-1)
+    fr = O.experts_rows_forward(x, ids, w1, w3, w2, emulate_bf16=True)
+    br = O.experts_rows_backward(fr, dy, w1, w3, w2, emulate_bf16=True)
+    assert torch.equal(fr["out"], fe["out"])
+    assert torch.equal(br["drows"], be["dx_expert"])
+    for n in ("dw1", "dw3", "dw2"):
+        assert torch.equal(br[n], be[n]), n
+
+
 # ----------------------------------------------------------------------------- block oracle
 def test_block_oracle_pieces():
     from oracle import block_oracle as B
@@ -285,6 +402,18 @@ def test_block_oracle_pieces():
     assert torch.allclose(q2[..., 0, :], q[..., 0, :]) and torch.allclose(k2[..., 0, :], k[..., 0, :])
     qa, _ = B.rope(2 * q, k)
     assert torch.allclose(qa, 2 * q2, atol=1e-6)
+    # element by element, as attn.py:53-54 and :61-63 write it for head_dim 4 at position p:
+    # cos = [c0, c0, c1, c1] (interleave-duplicated), rotate_half(q) = [-q2, -q3, q0, q1]
+    # (split in halves), so out = [q0 c0 - q2 s0, q1 c0 - q3 s0, q2 c1 + q0 s1, q3 c1 + q1 s1]
+    # with angle_i = p * theta^(-2i/4).  A layout that pairs (0,1),(2,3) or duplicates the angles
+    # as [c0, c1, c0, c1] gives different numbers.
+    import math
+    q4 = torch.tensor([[[[0.0, 0.0, 0.0, 0.0], [0.0, 0.0, 0.0, 0.0], [0.0, 0.0, 0.0, 0.0], [1.0, 2.0, 3.0, 4.0]]]])
+    r4, _ = B.rope(q4, q4)
+    a0, a1 = 3.0, 3.0 * 10000.0 ** (-0.5)
+    want = [1 * math.cos(a0) - 3 * math.sin(a0), 2 * math.cos(a0) - 4 * math.sin(a0),
+            3 * math.cos(a1) + 1 * math.sin(a1), 4 * math.cos(a1) + 2 * math.sin(a1)]
+    assert torch.allclose(r4[0, 0, 3], torch.tensor(want), atol=1e-5)
     # attention against the library's fused routine on the CPU
     nh, nkv, C = 4, 2, 32
     ws = [torch.randn(o, C, generator=g) * 0.2 for o in (C, C // 2, C // 2, C)]

@@ -30,31 +30,56 @@ __device__ __forceinline__ int wave_incl_scan(int v) {
 
 __device__ __forceinline__ int clamp_expert(int e, int E) { return e < 0 ? 0 : (e >= E ? E - 1 : e); }
 
+// whist [NW][E] per-wave histograms; wbad [NW] per-wave counts of ids outside [0, E) (such a
+// row is counted, and later placed, with the nearest valid expert so that every position of
+// the permutation is still written; the count is how the caller learns of it).
 __global__ __launch_bounds__(256) void hist_kernel(const int32_t* __restrict__ ids, int R, int E,
-                                                  int NW, int32_t* __restrict__ whist) {
+                                                  int NW, int32_t* __restrict__ whist,
+                                                  int32_t* __restrict__ wbad) {
   extern __shared__ int cnt[];  // [WAVES_PER_BLOCK][E]
   const int lane = lane_id(), wv = threadIdx.x / MOE_WAVE;
   const int w = blockIdx.x * WAVES_PER_BLOCK + wv;
   int* mine = cnt + wv * E;
   for (int e = lane; e < E; e += MOE_WAVE) mine[e] = 0;
   __syncthreads();
+  int bad = 0;
   if (w < NW) {
     const int base = w * ROWS_PER_WAVE;
 #pragma unroll
     for (int it = 0; it < ROWS_PER_WAVE / MOE_WAVE; ++it) {
       const int r = base + it * MOE_WAVE + lane;
-      if (r < R) atomicAdd(&mine[clamp_expert(ids[r], E)], 1);
+      if (r < R) {
+        const int e = ids[r];
+        bad += (e < 0 || e >= E) ? 1 : 0;
+        atomicAdd(&mine[clamp_expert(e, E)], 1);
+      }
     }
   }
   __syncthreads();
-  if (w < NW)
+  if (w < NW) {
     for (int e = lane; e < E; e += MOE_WAVE) whist[(size_t)w * E + e] = mine[e];
+#pragma unroll
+    for (int off = MOE_WAVE / 2; off > 0; off >>= 1) bad += __shfl_xor(bad, off, MOE_WAVE);
+    if (lane == 0) wbad[w] = bad;
+  }
 }
 
 // One wave per expert: exclusive scan down the column whist[:, e]; counts[e] = total.
+// Block E (one past the experts) adds up the per-wave counts of invalid ids into *bad_total
+// (when the caller asked for it).
 __global__ __launch_bounds__(64) void colscan_kernel(int32_t* __restrict__ whist, int NW, int E,
-                                                    int32_t* __restrict__ counts) {
+                                                    int32_t* __restrict__ counts,
+                                                    const int32_t* __restrict__ wbad,
+                                                    int32_t* __restrict__ bad_total) {
   const int e = blockIdx.x, lane = lane_id();
+  if (e == E) {
+    int sum = 0;
+    for (int w = lane; w < NW; w += MOE_WAVE) sum += wbad[w];
+#pragma unroll
+    for (int off = MOE_WAVE / 2; off > 0; off >>= 1) sum += __shfl_xor(sum, off, MOE_WAVE);
+    if (lane == 0) *bad_total = sum;
+    return;
+  }
   int running = 0;
   for (int base = 0; base < NW; base += MOE_WAVE) {
     const int w = base + lane;
@@ -351,29 +376,56 @@ extern "C" int moe_abi_version(void) { return 100; }
 extern "C" int64_t moe_dispatch_workspace_bytes(int64_t R, int64_t E) {
   if (R < 0 || E <= 0) return 0;
   const int64_t nw = (R + ROWS_PER_WAVE - 1) / ROWS_PER_WAVE;
-  return (nw > 0 ? nw : 1) * E * (int64_t)sizeof(int32_t);
+  return (nw > 0 ? nw : 1) * (E + 1) * (int64_t)sizeof(int32_t);  // [nw][E] histograms + [nw] invalid-id counts
+}
+
+namespace {
+
+int histogram_scan_impl(const int32_t* ids, int64_t R, int64_t E, int32_t* counts, int32_t* offs,
+                        int32_t* pos_to_row, int32_t* row_to_pos, int32_t* bad_ids, void* scratch,
+                        hipStream_t s) {
+  const int NW = (int)((R + ROWS_PER_WAVE - 1) / ROWS_PER_WAVE);
+  const int nblk = NW > 0 ? (NW + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK : 1;
+  const size_t lds = (size_t)WAVES_PER_BLOCK * E * sizeof(int);
+  int32_t* whist = (int32_t*)scratch;
+  int32_t* wbad = whist + (size_t)(NW > 0 ? NW : 1) * E;
+  if (NW > 0) {
+    hipLaunchKernelGGL(hist_kernel, dim3(nblk), dim3(256), lds, s, ids, (int)R, (int)E, NW, whist, wbad);
+  }
+  hipLaunchKernelGGL(colscan_kernel, dim3((unsigned)E + (bad_ids ? 1u : 0u)), dim3(64), 0, s, whist, NW,
+                     (int)E, counts, wbad, bad_ids);
+  hipLaunchKernelGGL(positions_kernel, dim3(nblk), dim3(256), lds, s, ids, (int)R, (int)E, NW,
+                     whist, counts, offs, pos_to_row, row_to_pos);
+  return moe_launch_status();
+}
+
+int histogram_scan_args(const int32_t* ids, int64_t R, int64_t E, const int32_t* counts,
+                        const int32_t* offs, const int32_t* pos_to_row, const int32_t* row_to_pos) {
+  if (!counts || !offs) return MOE_ERR_NULL;
+  if (R > 0 && (!ids || !pos_to_row || !row_to_pos)) return MOE_ERR_NULL;
+  if (R < 0 || E <= 0) return MOE_ERR_SHAPE;
+  if (E > MOE_MAX_EXPERTS || R > (int64_t)1 << 30) return MOE_ERR_LIMIT;
+  return 0;
+}
+
+}  // namespace
+
+extern "C" int moe_histogram_scan_checked(const int32_t* ids, int64_t R, int64_t E, int32_t* counts,
+                                          int32_t* offs, int32_t* pos_to_row, int32_t* row_to_pos,
+                                          int32_t* bad_ids, void* workspace, int64_t workspace_bytes,
+                                          void* stream) {
+  if (int rc = histogram_scan_args(ids, R, E, counts, offs, pos_to_row, row_to_pos)) return rc;
+  if (!workspace) return MOE_ERR_NULL;
+  if (workspace_bytes < moe_dispatch_workspace_bytes(R, E)) return MOE_ERR_WORKSPACE;
+  return histogram_scan_impl(ids, R, E, counts, offs, pos_to_row, row_to_pos, bad_ids, workspace,
+                             (hipStream_t)stream);
 }
 
 extern "C" int moe_histogram_scan(const int32_t* ids, int64_t R, int64_t E, int32_t* counts,
                                   int32_t* offs, int32_t* pos_to_row, int32_t* row_to_pos,
                                   void* workspace, int64_t workspace_bytes, void* stream) {
-  if (!counts || !offs || !workspace) return MOE_ERR_NULL;
-  if (R > 0 && (!ids || !pos_to_row || !row_to_pos)) return MOE_ERR_NULL;
-  if (R < 0 || E <= 0) return MOE_ERR_SHAPE;
-  if (E > MOE_MAX_EXPERTS || R > (int64_t)1 << 30) return MOE_ERR_LIMIT;
-  if (workspace_bytes < moe_dispatch_workspace_bytes(R, E)) return MOE_ERR_WORKSPACE;
-  hipStream_t s = (hipStream_t)stream;
-  const int NW = (int)((R + ROWS_PER_WAVE - 1) / ROWS_PER_WAVE);
-  const int nblk = NW > 0 ? (NW + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK : 1;
-  const size_t lds = (size_t)WAVES_PER_BLOCK * E * sizeof(int);
-  int32_t* whist = (int32_t*)workspace;
-  if (NW > 0) {
-    hipLaunchKernelGGL(hist_kernel, dim3(nblk), dim3(256), lds, s, ids, (int)R, (int)E, NW, whist);
-  }
-  hipLaunchKernelGGL(colscan_kernel, dim3((unsigned)E), dim3(64), 0, s, whist, NW, (int)E, counts);
-  hipLaunchKernelGGL(positions_kernel, dim3(nblk), dim3(256), lds, s, ids, (int)R, (int)E, NW,
-                     whist, counts, offs, pos_to_row, row_to_pos);
-  return moe_launch_status();
+  return moe_histogram_scan_checked(ids, R, E, counts, offs, pos_to_row, row_to_pos, nullptr, workspace,
+                                    workspace_bytes, stream);
 }
 
 extern "C" int moe_permute_fwd(const void* x, int x_dtype, const int32_t* pos_to_row, int64_t R,

@@ -223,7 +223,10 @@ def moe_ffn(x: torch.Tensor, logits: torch.Tensor, w1: torch.Tensor, w3: torch.T
             w2: torch.Tensor, k: int, bias: torch.Tensor | None = None, return_routing: bool = False,
             bf16_weights=None, accumulate_into_grad: bool = False):
     """out[t] = sum_j gate[t,j] * FFN_{e(t,j)}(x[t]).  x [T,H]; logits [T,E]; w1,w3 [E,I,H];
-    w2 [E,H,I].  `bias` (fp32 [E]) is added to the logits before selection only.
+    w2 [E,H,I].  `bias` (fp32 [E]) is added to the logits in fp32 and is part of them from
+    there on: both the selection and the softmax over the selected values see logit + bias
+    (a per-expert constant in the router, as benchmark config 2 specifies), and its gradient
+    is the column sum of dlogits.
     With `return_routing` also returns a dict of the integer routing tensors and gates.
     `bf16_weights`: bf16 copies of (w1, w3, w2) to compute with (None entries are cast here).
     `accumulate_into_grad`: w1, w3, w2 must be leaf tensors; see the module docstring."""
@@ -236,6 +239,9 @@ def moe_ffn(x: torch.Tensor, logits: torch.Tensor, w1: torch.Tensor, w3: torch.T
         return out, {"ids": ids, "gates": gates, "counts": counts, "offs": offs,
                      "pos_to_row": pos_to_row, "row_to_pos": row_to_pos}
     return out
+
+
+_ROUTING_NAMES = ("ids", "gates", "counts", "offs", "pos_to_row", "row_to_pos")
 
 
 class _PreNormMoE(torch.autograd.Function):
@@ -279,11 +285,12 @@ class _PreNormMoE(torch.autograd.Function):
         ctx.x_dtype, ctx.x_shape = x.dtype, x.shape
         ctx.nw_dtype = norm_w.dtype if ctx.has_norm else None
         ctx.wr_dtype, ctx.w_dtype = wr.dtype, w1.dtype
+        ctx.mark_non_differentiable(ids, gates, counts, offs, pos_to_row, row_to_pos)
         ctx.set_materialize_grads(False)
-        return out, logits
+        return out, logits, ids, gates, counts, offs, pos_to_row, row_to_pos
 
     @staticmethod
-    def backward(ctx, dout, dlogits_ext):
+    def backward(ctx, dout, dlogits_ext, *unused):
         (x, nw, rstd, xn, wrb, xp, g, u, act, gates, ids, offs, pos_to_row, row_to_pos,
          w1b, w3b, w2b) = ctx.saved_tensors
         k, E = ctx.k, ctx.E
@@ -320,7 +327,8 @@ class _PreNormMoE(torch.autograd.Function):
 
 def prenorm_moe(x: torch.Tensor, norm_weight: torch.Tensor, router_weight: torch.Tensor,
                 w1: torch.Tensor, w3: torch.Tensor, w2: torch.Tensor, k: int, eps: float = 1e-6,
-                add_residual: bool = True, bf16_weights=None, accumulate_into_grad: bool = False):
+                add_residual: bool = True, bf16_weights=None, accumulate_into_grad: bool = False,
+                return_routing: bool = False):
     """(x + MoE(RMSNorm(x)), router logits) for x [T,H]: model/gpt.py:32-33 with
     model/modules/norm.py:14-19 and model/modules/mlp.py:95-169 in one differentiable call.
     Router logits are bf16 (what the reference produces under its bf16 autocast); the output
@@ -328,23 +336,30 @@ def prenorm_moe(x: torch.Tensor, norm_weight: torch.Tensor, router_weight: torch
     grad_params = None
     if accumulate_into_grad:
         grad_params = tuple(w if (w.requires_grad and w.is_leaf) else None for w in (w1, w3, w2))
-    return _PreNormMoE.apply(x, norm_weight, router_weight, w1, w3, w2, float(eps), k, None, bf16_weights,
-                             grad_params, add_residual)
+    res = _PreNormMoE.apply(x, norm_weight, router_weight, w1, w3, w2, float(eps), k, None, bf16_weights,
+                            grad_params, add_residual)
+    if return_routing:
+        return res[0], res[1], dict(zip(_ROUTING_NAMES, res[2:]))
+    return res[0], res[1]
 
 
 def routed_moe(x: torch.Tensor, router_weight: torch.Tensor, w1: torch.Tensor, w3: torch.Tensor,
                w2: torch.Tensor, k: int, bias: torch.Tensor | None = None, bf16_weights=None,
-               accumulate_into_grad: bool = False):
+               accumulate_into_grad: bool = False, return_routing: bool = False):
     """(MoE(x), router logits) for x [T,H]: `router_linear` and `moe_ffn` as one autograd node
     (mlp.py:100-167), so that the two gradient contributions to x (expert path, router path)
     are summed inside the k-row-sum kernel.  The router product is a bf16 library product
     whatever the dtypes (the reference's behaviour under its bf16 autocast); the output has
-    the dtype of x."""
+    the dtype of x.  With `return_routing` a dict of the integer routing tensors and gates is
+    returned as a third value."""
     grad_params = None
     if accumulate_into_grad:
         grad_params = tuple(w if (w.requires_grad and w.is_leaf) else None for w in (w1, w3, w2))
-    return _PreNormMoE.apply(x, None, router_weight, w1, w3, w2, 0.0, k, bias, bf16_weights, grad_params,
-                             False)
+    res = _PreNormMoE.apply(x, None, router_weight, w1, w3, w2, 0.0, k, bias, bf16_weights, grad_params,
+                            False)
+    if return_routing:
+        return res[0], res[1], dict(zip(_ROUTING_NAMES, res[2:]))
+    return res[0], res[1]
 
 
 class _ExpertsRows(torch.autograd.Function):
@@ -355,7 +370,7 @@ class _ExpertsRows(torch.autograd.Function):
         rows = rows.contiguous()
         ids32 = ids.to(torch.int32).contiguous()
         w1b, w3b, w2b = (ops.cast_bf16(w.contiguous()) for w in (w1, w3, w2))
-        counts, offs, pos_to_row, row_to_pos = ops.histogram_scan(ids32, E)
+        counts, offs, pos_to_row, row_to_pos, bad = ops.histogram_scan(ids32, E, return_bad=True)
         xp = ops.permute_fwd(rows, pos_to_row, 1)
         train = any(ctx.needs_input_grad)
         g, u, act = ops.gemm_gateup(xp, w1b, w3b, offs, save_gu=train)
@@ -365,10 +380,10 @@ class _ExpertsRows(torch.autograd.Function):
             ctx.save_for_backward(xp, g, u, act, offs, pos_to_row, row_to_pos, w1b, w3b, w2b)
         ctx.x_dtype, ctx.w_dtype = rows.dtype, w1.dtype
         ctx.grad_params = grad_params
-        ctx.mark_non_differentiable(counts, offs, pos_to_row, row_to_pos)
+        ctx.mark_non_differentiable(counts, offs, pos_to_row, row_to_pos, bad)
         ctx.set_materialize_grads(False)
         ctx.out_shape = out.shape
-        return out, counts, offs, pos_to_row, row_to_pos
+        return out, counts, offs, pos_to_row, row_to_pos, bad
 
     @staticmethod
     def backward(ctx, dout, *unused):
@@ -387,13 +402,23 @@ class _ExpertsRows(torch.autograd.Function):
 
 
 def experts_rows(rows: torch.Tensor, ids: torch.Tensor, w1, w3, w2, return_routing: bool = False,
-                 accumulate_into_grad: bool = False):
+                 accumulate_into_grad: bool = False, check_ids: bool = False):
     """One rank's local expert share: rows [R,H] already dispatched to this rank, ids [R]
-    local expert index of each row -> FFN output rows in the same (arrival) order."""
+    local expert index of each row -> FFN output rows in the same (arrival) order.
+
+    ids must lie in [0, E).  The dispatch kernels count the ids that do not (and treat such a
+    row as belonging to the nearest valid expert, so nothing reads out of bounds); the count is
+    a device tensor, `bad_ids` in the routing dict, so the hot path never waits for it.  With
+    `check_ids` the call synchronises and raises ValueError if the count is not zero."""
     grad_params = None
     if accumulate_into_grad:
         grad_params = tuple(w if (w.requires_grad and w.is_leaf) else None for w in (w1, w3, w2))
-    out, counts, offs, pos_to_row, row_to_pos = _ExpertsRows.apply(rows, ids, w1, w3, w2, grad_params)
+    out, counts, offs, pos_to_row, row_to_pos, bad = _ExpertsRows.apply(rows, ids, w1, w3, w2, grad_params)
+    if check_ids:
+        n = int(bad.item())
+        if n:
+            raise ValueError(f"experts_rows: {n} of {ids.numel()} expert ids lie outside [0, {w1.shape[0]})")
     if return_routing:
-        return out, {"counts": counts, "offs": offs, "pos_to_row": pos_to_row, "row_to_pos": row_to_pos}
+        return out, {"counts": counts, "offs": offs, "pos_to_row": pos_to_row, "row_to_pos": row_to_pos,
+                     "bad_ids": bad}
     return out

@@ -50,8 +50,10 @@ def router_topk_bwd(gates, dgates, ids, T: int, E: int, k: int, dtype: torch.dty
     return dlogits
 
 
-def histogram_scan(ids: torch.Tensor, E: int):
-    """ids int32 [R] -> counts int32 [E], offs int32 [E+1], pos_to_row, row_to_pos int32 [R]."""
+def histogram_scan(ids: torch.Tensor, E: int, return_bad: bool = False):
+    """ids int32 [R] -> counts int32 [E], offs int32 [E+1], pos_to_row, row_to_pos int32 [R].
+    With `return_bad` a fifth tensor (int32 [1], on the device) holds the number of ids outside
+    [0, E); reading it is the caller's business (it costs a synchronisation)."""
     R = ids.numel()
     dev = ids.device
     L = _lib.load()
@@ -61,8 +63,11 @@ def histogram_scan(ids: torch.Tensor, E: int):
     offs = torch.empty(E + 1, dtype=torch.int32, device=dev)
     pos_to_row = torch.empty(R, dtype=torch.int32, device=dev)
     row_to_pos = torch.empty(R, dtype=torch.int32, device=dev)
-    L.call("moe_histogram_scan", _p(ids), R, E, _p(counts), _p(offs), _p(pos_to_row),
-           _p(row_to_pos), _p(ws), ws.numel(), _stream())
+    bad = torch.empty(1, dtype=torch.int32, device=dev) if return_bad else None
+    L.call("moe_histogram_scan_checked", _p(ids), R, E, _p(counts), _p(offs), _p(pos_to_row),
+           _p(row_to_pos), _p(bad), _p(ws), ws.numel(), _stream())
+    if return_bad:
+        return counts, offs, pos_to_row, row_to_pos, bad
     return counts, offs, pos_to_row, row_to_pos
 
 
