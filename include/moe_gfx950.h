@@ -21,8 +21,8 @@
  *   - Alignment: H and I must be multiples of 8 (rows are moved as 16-byte vectors) and
  *     every pointer 16-byte aligned.
  *   - Limits: E <= MOE_MAX_EXPERTS for routing and dispatch, E <= 1024 for the GEMMs,
- *     k <= MOE_MAX_TOPK, R <= 2^30, and R * max(H, I) < 2^31 elements (one expert's rows
- *     are walked with a 32-bit byte offset).
+ *     k <= MOE_MAX_TOPK, R <= 2^30, H and I <= 65536, and fewer than 2^31 output tiles per
+ *     GEMM ((R/256 + E + 1) * ceil(max(H, I)/128)).  Buffers may exceed 4 GiB.
  */
 #ifndef MOE_GFX950_H
 #define MOE_GFX950_H

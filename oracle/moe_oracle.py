@@ -251,7 +251,8 @@ def moe_backward(fwd: dict, dy: torch.Tensor, wr: torch.Tensor, w1: torch.Tensor
     if emulate_bf16:
         dlogits_used = _maybe_round(dlogits, True)
     dwr = dlogits_used.t() @ x2
-    dx_router = dlogits_used @ wrc
+    # (the router path's input gradient is a bf16 library product on the device)
+    dx_router = _maybe_round(dlogits_used @ wrc, emulate_bf16)
     return {"dyp": dyp, "dgates": dgates, "dg": dg, "du": du, "dxp": dxp, "dw1": dw1,
             "dw3": dw3, "dw2": dw2, "dx_expert": dx_expert, "dsel": dsel, "dlogits": dlogits,
             "dwr": dwr, "dx_router": dx_router, "dx": (dx_expert + dx_router).reshape(dy.shape),

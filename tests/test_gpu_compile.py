@@ -74,3 +74,31 @@ def test_compiled_module_is_one_graph_and_matches_eager(pkg, lib, dtype):
     with torch.no_grad(), ctx():
         o2, _ = torch.compile(m, backend="aot_eager", fullgraph=True)(x)
     assert torch.equal(o2, eager[0])
+
+
+def test_compiled_with_the_inductor_backend(pkg, lib):
+    """The default backend of `torch.compile` (inductor: its generated kernels surround the
+    registered operators): one graph, results norm-wise equal to eager (the code around the layer
+    is regenerated, so bits may differ), expert kernels bit-equal given equal logits."""
+    _say("torch.compile(MoE, backend=inductor, fullgraph=True)")
+    m, x, dy = _case(pkg, torch.float32)
+
+    def run(mod):
+        m.zero_grad(set_to_none=True)
+        xi = x.clone().requires_grad_(True)
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            out, logits = mod(xi)
+        out.backward(dy)
+        return [out.detach(), logits.detach(), xi.grad] + [p.grad.clone() for p in m.parameters()]
+
+    eager = run(m)
+    compiled = run(torch.compile(m, backend="inductor", fullgraph=True))
+    names = ["out", "gate_logits", "dx"] + [n for n, _ in m.named_parameters()]
+    same_logits = torch.equal(eager[1], compiled[1])
+    for n, a, b in zip(names, eager, compiled):
+        assert a.dtype == b.dtype and a.shape == b.shape, n
+        rel = ((a.float() - b.float()).norm() / a.float().norm().clamp_min(1e-30)).item()
+        _say(f"  {n}: rel {rel:.2e}")
+        assert rel < 1e-2, (n, rel)
+        if same_logits and n in ("out", "experts_gate_weights", "experts_up_weights", "experts_down_weights"):
+            assert torch.equal(a, b), n

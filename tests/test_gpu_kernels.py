@@ -367,6 +367,52 @@ def test_gate_gradients_from_the_dgrad_down_kernel(ops, R, H, I, E, empty):
     assert torch.equal(again, dgates)  # reproducible
 
 
+def test_grouped_gemms_on_buffers_beyond_4_gib(ops):
+    """Row buffers larger than 4 GiB, one expert owning more than 4 GiB of them: the rows on
+    both sides of the 2^32-byte mark (row 2^20 at 4096 bytes per row) and the last rows must come
+    out as they do at the start of the buffer, for every grouped product."""
+    _say("grouped GEMMs, R*H*2 > 2^32")
+    H, I, E = 2048, 16, 3
+    n0 = (1 << 20) + 2000
+    R = n0 + 900
+    offs = torch.tensor([0, n0, n0, R], dtype=torch.int32).cuda()   # expert 1 has no rows
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    xp = torch.randn(R, H, device="cuda", generator=gen).to(torch.bfloat16)
+    assert xp.numel() * 2 > 1 << 32
+    w1 = (torch.randn(E, I, H, device="cuda", generator=gen) * 0.05).to(torch.bfloat16)
+    w3 = (torch.randn(E, I, H, device="cuda", generator=gen) * 0.05).to(torch.bfloat16)
+    w2 = (torch.randn(E, H, I, device="cuda", generator=gen) * 0.05).to(torch.bfloat16)
+    windows = [(0, 300), ((1 << 20) - 300, (1 << 20) + 300), (n0 - 200, n0), (n0, n0 + 200), (R - 150, R)]
+    expert_of = lambda a: 0 if a < n0 else 2
+
+    g, u, act = ops.gemm_gateup(xp, w1, w3, offs, save_gu=True)
+    y = ops.gemm_down(act, w2, offs)
+    dg, du = ops.gemm_dgrad_down(xp, w2, g, u, offs)          # xp doubles as the incoming gradient rows
+    dxp = ops.gemm_dgrad_gateup(dg, du, w1, w3, offs)
+    for a, b in windows:
+        e = expert_of(a)
+        xs = xp[a:b].float()
+        gr, ur = xs @ w1[e].float().t(), xs @ w3[e].float().t()
+        assert _close(g[a:b], gr) and _close(u[a:b], ur) and _close(act[a:b], torch.nn.functional.silu(gr) * ur), (a, b)
+        assert _close(y[a:b], act[a:b].float() @ w2[e].float().t()), (a, b)
+        dact = xs @ w2[e].float()
+        gf, uf = g[a:b].float(), u[a:b].float()
+        sg = torch.sigmoid(gf)
+        assert _close(dg[a:b], dact * uf * (sg * (1 + gf * (1 - sg)))) and _close(du[a:b], dact * gf * sg), (a, b)
+        assert _close(dxp[a:b], dg[a:b].float() @ w1[e].float() + du[a:b].float() @ w3[e].float()), (a, b)
+    # weight gradient: a contraction that runs across the 4 GiB mark (fixed order, fp32 sums)
+    dw = ops.gemm_wgrad(act, xp, offs, E, torch.float32)        # [E, I, H]
+    for e, (a, b) in ((0, (0, n0)), (2, (n0, R))):
+        ref = torch.zeros(I, H, device="cuda")
+        for c in range(a, b, 1 << 18):
+            d = min(b, c + (1 << 18))
+            ref += act[c:d].float().t() @ xp[c:d].float()
+        rel = ((dw[e] - ref).norm() / ref.norm()).item()
+        _say(f"  dw[{e}] rel {rel:.2e}")
+        assert rel < 1e-3
+    assert not dw[1].any()
+
+
 def test_gemm_zero_rows(ops):
     E, H, I = 4, 64, 32
     offs = torch.zeros(E + 1, dtype=torch.int32).cuda()

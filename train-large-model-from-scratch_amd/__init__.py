@@ -1,5 +1,5 @@
 """MI355X-native MoE expert path (drop-in for the reference's model/modules/mlp.py::MoE)."""
-from . import configs, lib, ops, parallel_state  # noqa: F401
+from . import configs, lib, ops, parallel_state, profile  # noqa: F401
 from .config import ModelConfig  # noqa: F401
 from .functional import experts_rows, moe_ffn, prenorm_moe, routed_moe, router_linear  # noqa: F401
 from .moe import MoE  # noqa: F401

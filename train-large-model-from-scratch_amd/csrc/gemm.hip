@@ -922,9 +922,11 @@ int check_common(const int32_t* offs, int64_t E, int64_t R, int64_t H, int64_t I
   if (!offs) return MOE_ERR_NULL;
   if (E <= 0 || R < 0 || H <= 0 || I <= 0 || (H % 8) || (I % 8)) return MOE_ERR_SHAPE;
   if (E > GEMM_MAX_E || R > (int64_t)1 << 30 || H > (1 << 16) || I > (1 << 16)) return MOE_ERR_LIMIT;
-  // the kernels walk one expert's rows with a 32-bit byte offset, and one expert may own
-  // all R rows
-  if (R * (H > I ? H : I) * 2 >= ((int64_t)1 << 32)) return MOE_ERR_LIMIT;
+  // Row and column positions are 64-bit wherever they are multiplied by a row length; what is
+  // 32-bit is the per-lane offset inside one tile's window (at most 256 rows of 65536 elements)
+  // and the tile index: rows / 256 + E row slots times the column tiles of the widest output.
+  const int64_t widest = H > I ? H : I;
+  if ((R / 256 + E + 1) * ((widest + 127) / 128) >= ((int64_t)1 << 31)) return MOE_ERR_LIMIT;
   return 0;
 }
 

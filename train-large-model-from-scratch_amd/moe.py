@@ -17,14 +17,18 @@ from .functional import moe_ffn, prenorm_moe, routed_moe, router_linear
 
 # Number of optimizer steps taken in this process, counted by a global post-step hook of
 # torch.optim: one of the signs that master weights may have changed (see MoE._bf16_operands).
+# The hook is installed when the first MoE that caches its weight copies is built, not at import.
 _optimizer_steps = [0]
+_hook_handle = []
 
 
 def _count_optimizer_step(optimizer, args, kwargs):
     _optimizer_steps[0] += 1
 
 
-register_optimizer_step_post_hook(_count_optimizer_step)
+def _install_step_counter():
+    if not _hook_handle:
+        _hook_handle.append(register_optimizer_step_post_hook(_count_optimizer_step))
 
 
 class MoE(nn.Module):
@@ -57,6 +61,13 @@ class MoE(nn.Module):
         self.experts_down_weights = nn.Parameter(torch.empty(E, H, I, device=self.device))
         self.experts_act_fn = nn.SiLU()
         self._shadow = {}  # name -> (key of the master's state, bf16 copy); not part of state_dict
+        # False: cast the fp32 masters in every forward, as the reference does (no cached copies,
+        # nothing that a write through `.data` could leave stale).
+        self.cache_bf16_weights = True
+        # True: before every use of a cached copy, 64 of its elements are compared with the
+        # master (one small gather and a host synchronisation per stack) and a stale copy raises.
+        self.verify_weight_cache = False
+        _install_step_counter()
         # Opt-in: expert weight gradients are added to `.grad` by the kernel that computes them
         # instead of by autograd (saves a pass over them per gradient-accumulation micro-step;
         # hooks on these three parameters then do not run, see functional.py).
@@ -98,8 +109,10 @@ class MoE(nn.Module):
             broadcasts through `p.data` (distributed_optimizer.py:85-94, :119), which the
             version counter does not see,
           - the master's storage or device.
-        Writes through `.data` with no optimizer step in between are the one case this cannot
-        see; `invalidate_weight_cache()` is there for them.  The copies are handed to the
+        Writes through `.data` with no `torch.optim` step in between (an EMA swap, a manual
+        `p.data.copy_`, an optimizer that is not a `torch.optim.Optimizer`) are the one case this
+        cannot see: `invalidate_weight_cache()` is there for them, `cache_bf16_weights = False`
+        turns the cache off, and `verify_weight_cache = True` detects a stale copy.  The copies are handed to the
         expert function together with the masters: the masters receive the gradients."""
         out = []
         for name in ("experts_gate_weights", "experts_up_weights", "experts_down_weights"):
@@ -107,11 +120,21 @@ class MoE(nn.Module):
             if w.dtype == torch.bfloat16:
                 out.append(None)
                 continue
+            if not self.cache_bf16_weights:
+                out.append(None)  # the expert function casts
+                continue
             key = (w._version, _optimizer_steps[0], w.data_ptr(), w.device)
             held = self._shadow.get(name)
             if held is None or held[0] != key:
                 held = (key, ops.cast_bf16(w.detach().contiguous()))
                 self._shadow[name] = held
+            elif self.verify_weight_cache:
+                idx = torch.randint(0, w.numel(), (64,), device=w.device)
+                if not torch.equal(w.detach().reshape(-1)[idx].to(torch.bfloat16), held[1].reshape(-1)[idx]):
+                    raise RuntimeError(
+                        f"MoE: the cached bf16 copy of {name} no longer matches its fp32 master (the master "
+                        "was rewritten without an optimizer step or a version bump); call "
+                        "invalidate_weight_cache() after such writes or set cache_bf16_weights = False")
             out.append(held[1])
         return out
 
