@@ -86,6 +86,21 @@ int moe_histogram_scan_checked(const int32_t* ids, int64_t R, int64_t E, int32_t
                                int32_t* bad_ids, void* workspace, int64_t workspace_bytes,
                                void* stream);
 
+/* moe_histogram_scan_checked without a workspace argument and without any allocation.  It has no
+ * counterpart in the reference; it is for callers that cannot allocate device memory at the
+ * point of the call (code under HIP graph capture, serving loops with a frozen memory plan,
+ * harnesses that forbid hipMalloc).  The per-wave histograms go to a fixed array of
+ * moe_static_scratch_bytes() (4 MiB) that the library holds in every GPU's memory until the
+ * process ends; MOE_ERR_WORKSPACE if moe_dispatch_workspace_bytes(R, E) exceeds it (i.e.
+ * ceil(R/256) * (E+1) * 4 > 4 MiB: up to 1 M routed rows at 512 experts, 16 M at 64).  All calls
+ * on one GPU share that array: two such calls that overlap in time on one GPU (different
+ * streams, or graphs replayed concurrently) race; calls ordered on one stream do not.  Results
+ * are bit-identical to moe_histogram_scan_checked. */
+int64_t moe_static_scratch_bytes(void);
+int moe_histogram_scan_static(const int32_t* ids, int64_t R, int64_t E, int32_t* counts,
+                              int32_t* offs, int32_t* pos_to_row, int32_t* row_to_pos,
+                              int32_t* bad_ids, void* stream);
+
 /* Replaces `repeat_interleave(k)` + the two row gathers (mlp.py:104, 108, 124):
  * xp[pos,:] = bf16(x[pos_to_row[pos] / k, :]).  x [T,H] (x_dtype), xp bf16 [R,H]. */
 int moe_permute_fwd(const void* x, int x_dtype, const int32_t* pos_to_row, int64_t R,

@@ -1,0 +1,69 @@
+"""The dispatch entry point that allocates nothing (`moe_histogram_scan_static`): called through
+the C ABI with caller-owned inputs and outputs, its results must equal, bit for bit, those of
+the entry point that takes a workspace, on two calls in a row (the second with a smaller input,
+so that the scratch array still holds the first call's histograms), and sizes beyond the fixed
+scratch must be refused."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _outputs(R, E):
+    i32 = lambda n: torch.full((n,), -7, dtype=torch.int32, device="cuda")
+    return i32(E), i32(E + 1), i32(R), i32(R), i32(1)
+
+
+def _call_static(L, ids, E):
+    R = ids.numel()
+    counts, offs, p2r, r2p, bad = _outputs(R, E)
+    stream = torch.cuda.current_stream().cuda_stream
+    before = torch.cuda.memory_stats()["allocation.all.allocated"]
+    L.call("moe_histogram_scan_static", ids.data_ptr(), R, E, counts.data_ptr(), offs.data_ptr(),
+           p2r.data_ptr(), r2p.data_ptr(), bad.data_ptr(), stream)
+    assert torch.cuda.memory_stats()["allocation.all.allocated"] == before  # nothing came from torch's allocator
+    return counts, offs, p2r, r2p, bad
+
+
+def _call_workspace(L, ids, E):
+    R = ids.numel()
+    counts, offs, p2r, r2p, bad = _outputs(R, E)
+    nbytes = L.cdll.moe_dispatch_workspace_bytes(R, E)
+    ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device="cuda")
+    L.call("moe_histogram_scan_checked", ids.data_ptr(), R, E, counts.data_ptr(), offs.data_ptr(),
+           p2r.data_ptr(), r2p.data_ptr(), bad.data_ptr(), ws.data_ptr(), ws.numel(),
+           torch.cuda.current_stream().cuda_stream)
+    return counts, offs, p2r, r2p, bad
+
+
+def test_static_scratch_dispatch_equals_the_workspace_entry(pkg, lib):
+    assert torch.cuda.is_available()
+    L = lib
+    assert L.cdll.moe_static_scratch_bytes() == 4 << 20
+    rng = np.random.default_rng(5)
+    # two calls in a row on the same stream; the second is smaller and has fewer experts, so
+    # its histograms overlay a part of what the first left in the scratch array
+    cases = [(131072, 64), (5000, 16), (70000, 512), (300, 9), (0, 4), (1, 1)]
+    for R, E in cases:
+        print("static dispatch R", R, "E", E, flush=True)
+        ids_np = rng.integers(0, E, size=R)
+        if R >= 300:
+            ids_np[rng.choice(R, size=3, replace=False)] = E + 5   # invalid ids are counted the same way
+        ids = torch.from_numpy(ids_np.astype(np.int32)).cuda()
+        got = _call_static(L, ids, E)
+        want = _call_workspace(L, ids, E)
+        torch.cuda.synchronize()
+        for a, b, name in zip(got, want, ("counts", "offs", "pos_to_row", "row_to_pos", "bad_ids")):
+            assert torch.equal(a, b), (R, E, name)
+        assert got[4].item() == (3 if R >= 300 else 0)
+        assert got[1][-1].item() == R
+    # beyond the fixed scratch: refused, nothing enqueued
+    R, E = 300 * 256 * 8, 512   # ceil(R/256) * (E+1) * 4 bytes > 4 MiB
+    assert L.cdll.moe_dispatch_workspace_bytes(R, E) > L.cdll.moe_static_scratch_bytes()
+    ids = torch.zeros(R, dtype=torch.int32, device="cuda")
+    counts, offs, p2r, r2p, bad = _outputs(R, E)
+    with pytest.raises(pkg.lib.MoELibError, match="MOE_ERR_WORKSPACE"):
+        L.call("moe_histogram_scan_static", ids.data_ptr(), R, E, counts.data_ptr(), offs.data_ptr(),
+               p2r.data_ptr(), r2p.data_ptr(), bad.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    assert (counts == -7).all()

@@ -11,6 +11,8 @@
 //      ballots, and gives row r the position offs[e] + rows-of-e-in-earlier-waves +
 //      rows-of-e-earlier-in-this-wave -- i.e. the stable order -- writing both the
 //      permutation and its inverse.
+#include <mutex>
+
 #include "common.h"
 
 namespace {
@@ -426,6 +428,55 @@ extern "C" int moe_histogram_scan(const int32_t* ids, int64_t R, int64_t E, int3
                                   void* workspace, int64_t workspace_bytes, void* stream) {
   return moe_histogram_scan_checked(ids, R, E, counts, offs, pos_to_row, row_to_pos, nullptr, workspace,
                                     workspace_bytes, stream);
+}
+
+// ---- the dispatch entry that allocates nothing -----------------------------------------------
+// The per-wave histograms live in a fixed array in device memory that is part of the loaded
+// code object: every GPU the library runs on holds its own copy at its own address until the
+// process ends.  In host code the array's name is only a handle for the runtime; the address
+// kernels can use is asked for once per device and kept.
+#define MOE_STATIC_SCRATCH_BYTES (4 << 20)
+static __device__ __align__(256) unsigned char scratch[MOE_STATIC_SCRATCH_BYTES];
+
+namespace {
+
+constexpr int MAX_DEVICES = 64;
+void* scratch_of_device[MAX_DEVICES];  // device address of `scratch` on each GPU, 0 = not asked yet
+std::mutex scratch_mutex;
+
+// Device address of `scratch` on the current device (no allocation: a symbol lookup).
+int static_scratch(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= MAX_DEVICES) return MOE_ERR_LIMIT;
+  std::lock_guard<std::mutex> lock(scratch_mutex);
+  if (!scratch_of_device[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (!ptr) return MOE_ERR_NULL;
+    scratch_of_device[dev] = ptr;
+  }
+  *out = scratch_of_device[dev];
+  return 0;
+}
+
+}  // namespace
+
+extern "C" int64_t moe_static_scratch_bytes(void) { return MOE_STATIC_SCRATCH_BYTES; }
+
+extern "C" int moe_histogram_scan_static(const int32_t* ids, int64_t R, int64_t E, int32_t* counts,
+                                         int32_t* offs, int32_t* pos_to_row, int32_t* row_to_pos,
+                                         int32_t* bad_ids, void* stream) {
+  if (int rc = histogram_scan_args(ids, R, E, counts, offs, pos_to_row, row_to_pos)) return rc;
+  if (moe_dispatch_workspace_bytes(R, E) > MOE_STATIC_SCRATCH_BYTES) return MOE_ERR_WORKSPACE;
+  void* ptr = nullptr;
+  if (int rc = static_scratch(&ptr)) return rc;
+  // every word of the scratch that is read was written by this call's first kernel, so what
+  // an earlier call left behind needs no clearing
+  return histogram_scan_impl(ids, R, E, counts, offs, pos_to_row, row_to_pos, bad_ids, ptr,
+                             (hipStream_t)stream);
 }
 
 extern "C" int moe_permute_fwd(const void* x, int x_dtype, const int32_t* pos_to_row, int64_t R,
