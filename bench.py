@@ -53,9 +53,27 @@ def _event_time_ms(torch, fn, iters, warmup):
     return s.elapsed_time(e) / iters
 
 
-def bench_block(args, torch, P, dev):
+def _moe_dominant_kernel(torch, P, s, x_bf16, wr_bf16, ws_bf16):
+    """HIP-event duration of the gate/up grouped GEMM (the kernel with the largest share of the
+    layer) on the layer's own routing of `x_bf16`: the `roofline` object of a configuration."""
+    ops = P.ops
+    with torch.no_grad():
+        logits = x_bf16 @ wr_bf16.t()
+        ids, _ = ops.router_topk(logits, s.k, None)
+        _, offs, p2r, r2p = ops.histogram_scan(ids, s.E)
+        xp = ops.permute_fwd(x_bf16, p2r, s.k, r2p)
+        ms = _event_time_ms(torch, lambda: ops.gemm_gateup(xp, ws_bf16[0], ws_bf16[1], offs, True), 10, 2)
+    fl = 4 * s.R * s.H * s.I
+    return {"kernel": "gemm_gateup_swiglu_fwd", "bound": "mfma", "achieved": round(fl / ms / 1e9, 1),
+            "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(fl / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
+            "traffic": None, "ms": round(ms, 4)}
+
+
+def bench_block(args, torch, P, dev, steps=None, warmup=None, cpu=True):
     """Configuration 5: one GPT-MoE block (RMSNorm, GQA attention, MoE) forward+backward under
     bf16 autocast with fp32 parameters; reports tokens/s and the MoE's share of the time."""
+    steps = steps or args.steps
+    warmup = args.warmup if warmup is None else warmup
     s = P.configs.SHAPES[5]
     B, T = 2, 4096
     cfg = P.ModelConfig(hidden_size=s.H, num_attention_heads=32, num_key_value_heads=8, num_experts=s.E,
@@ -78,14 +96,14 @@ def bench_block(args, torch, P, dev):
         out.backward(dy)
 
     def timed():
-        for _ in range(args.warmup):
+        for _ in range(warmup):
             step()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(args.steps):
+        for _ in range(steps):
             step()
         torch.cuda.synchronize()
-        return (time.perf_counter() - t0) * 1e3 / args.steps
+        return (time.perf_counter() - t0) * 1e3 / steps
 
     # the caller as the reference writes it (gpt.py:32-33: norm, layer, residual add as three
     # calls), then with the norm and the residual add inside the layer's call
@@ -102,11 +120,38 @@ def bench_block(args, torch, P, dev):
             o = blk.mlp(moe_in)[0]
         o.backward(dy)
 
-    moe_ms = _event_time_ms(torch, moe_step, max(args.steps // 2, 3), 2)
+    moe_ms = _event_time_ms(torch, moe_step, max(steps // 2, 3), 2)
     flops = P.configs.gemm_flops(s)
-    line = {
+    bf = torch.bfloat16
+    m = blk.mlp
+    wb = [w.detach().to(bf) for w in (m.experts_gate_weights, m.experts_up_weights, m.experts_down_weights)]
+    x2 = moe_in.detach().reshape(B * T, s.H).to(bf)
+    roofline = _moe_dominant_kernel(torch, P, s, x2, m.router.weight.detach().to(bf), wb)
+    cpu_rec = None
+    if cpu:
+        # the oracle's per-expert loop on the rows the MoE received inside the block (1/4 of them)
+        from oracle import moe_oracle as O
+        ncores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
+        torch.set_num_threads(ncores)
+        n = B * T // 4
+        xc = x2[:n].cpu()
+        wc = [w.cpu().float() for w in wb]
+        wrc = m.router.weight.detach().to(bf).cpu().float()
+        dyc = dy.reshape(B * T, s.H)[:n].cpu()
+        t0 = time.perf_counter()
+        f = O.moe_forward(xc, wrc, *wc, s.k, logits_dtype=bf)
+        O.moe_backward(f, dyc, wrc, *wc)
+        dt = time.perf_counter() - t0
+        cpu_rec = {"value": round(n / dt, 1), "unit": "tokens/s", "cores": ncores, "kind": "port",
+                   "sample": f"MoE part only (oracle per-expert loop, fp32 math on the bf16 rows the layer received in "
+                             f"the block), {n} of {B * T} tokens, one timed pass of {dt:.2f} s; attention and norms "
+                             f"are stock torch on both sides and are not in the sample",
+                   "moe_tflops": round(18 * n * s.k * s.H * s.I / dt / 1e12, 4)}
+    del blk, wte
+    torch.cuda.empty_cache()
+    return {
         "metric": "gpt_moe_block_fwd_bwd_tokens_per_s", "value": round(B * T / (ms * 1e-3), 1), "unit": "tokens/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": s.name + " inside one GPT-MoE block (RMSNorm, GQA 32/8 heads x 64, seq 4096, batch 2), "
                                "fp32 parameters under bf16 autocast, ln_2 and the residual add inside the layer's call "
@@ -114,10 +159,129 @@ def bench_block(args, torch, P, dev):
         "ms_per_step_separate_norm_and_residual": round(ms_separate, 4),
         "moe_ms": round(moe_ms, 4), "moe_share_of_block_time": round(moe_ms / ms, 4),
         "moe_gemm_tflops": round(flops / moe_ms / 1e9, 1),
-        "roofline": None, "cpu_baseline": None,
+        "roofline": roofline, "cpu_baseline": cpu_rec,
     }
-    print(json.dumps(line), flush=True)
-    return 0
+
+
+def time_layer_config(P, torch, dev, cfg_id, steps, warmup):
+    """ms per step of one benchmark configuration (1, 2, 3 or 4) through the entry the module
+    uses (`routed_moe`; `experts_rows` for the post-dispatch configuration 4)."""
+    inp = P.configs.make_inputs(cfg_id)
+    s = inp["shape"]
+    if s.rows_entry:
+        x = inp["x"].to(dev).requires_grad_(True)
+        ids = inp["ids"].to(dev)
+        ws = [inp[n].to(dev).requires_grad_(True) for n in ("w1", "w3", "w2")]
+        dy = inp["dy"].to(dev)
+        leaves = (x, *ws)
+
+        def step():
+            for t in leaves:
+                t.grad = None
+            P.experts_rows(x, ids, *ws).backward(dy)
+    else:
+        x = inp["x"].to(dev).requires_grad_(s.backward)
+        wr = inp["wr"].to(dev).requires_grad_(s.backward)
+        ws = [inp[n].to(dev).requires_grad_(s.backward) for n in ("w1", "w3", "w2")]
+        dy = inp["dy"].to(dev) if s.backward else None
+        bias = inp["bias"].to(dev) if "bias" in inp else None
+        leaves = (x, wr, *ws)
+
+        def step():
+            for t in leaves:
+                t.grad = None
+            out, _ = P.routed_moe(x, wr, *ws, s.k, bias=bias)
+            if s.backward:
+                out.backward(dy)
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    flops = P.configs.gemm_flops(s)
+    return {"config": cfg_id, "workload": s.name, "entry": "experts_rows" if s.rows_entry else "routed_moe",
+            "ms_per_step": round(ms, 4), "tflops": round(flops / ms / 1e9, 1),
+            "mfma_peak_frac": round(flops / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
+            "tokens_per_s": round(s.T / (ms * 1e-3), 1), "steps": steps}
+
+
+def cpu_leg(P, torch, cfg_id, fraction=1.0):
+    """The oracle's per-expert loop (forward, and backward where the configuration has one) on
+    the host cores: the CPU baseline of a configuration."""
+    from oracle import moe_oracle as O
+    ncores = os.cpu_count() or 1
+    ncores = min(ncores, int(os.environ.get("OMP_NUM_THREADS", ncores)))
+    torch.set_num_threads(ncores)
+    cin = P.configs.make_inputs(cfg_id, scale_tokens=fraction)
+    s = cin["shape"]
+    w32 = [cin[n].float() for n in ("w1", "w3", "w2")]
+    t0 = time.perf_counter()
+    if s.rows_entry:
+        f = O.experts_rows_forward(cin["x"], cin["ids"].numpy(), *w32)
+        O.experts_rows_backward(f, cin["dy"].float(), *w32)
+        rows = cin["x"].shape[0]
+        toks = rows / s.k
+    else:
+        wr32 = cin["wr"].float()
+        f = O.moe_forward(cin["x"], wr32, *w32, s.k, bias=cin.get("bias"), logits_dtype=torch.bfloat16)
+        if s.backward:
+            O.moe_backward(f, cin["dy"].float(), wr32, *w32)
+        toks = cin["x"].shape[0]
+        rows = toks * s.k
+    dt = time.perf_counter() - t0
+    cflops = (18 if s.backward else 6) * rows * s.H * s.I
+    return {"value": round(cflops / dt / 1e12, 4), "unit": "TFLOP/s", "cores": ncores, "kind": "port",
+            "sample": f"oracle per-expert loop, fp32 math on the same bf16 inputs, {int(toks)} of {s.T} tokens "
+                      f"({rows} routed rows, all {s.E} experts), one timed pass of {dt:.2f} s",
+            "tokens_per_s": round(toks / dt, 1)}
+
+
+def module_config3(P, torch, dev, steps, warmup):
+    """Configuration 3 through the module as the reference's trainer calls it (trainer.py:209-216,
+    241-248): fp32 master weights and fp32 residual input under bf16 autocast, fp32 weight
+    gradients; a fresh step (gradients created) and a gradient-accumulation micro-step with the
+    weight-gradient kernel adding into `.grad`."""
+    s = P.configs.SHAPES[3]
+    inp = P.configs.make_inputs(3)
+    cfg = P.ModelConfig(hidden_size=s.H, num_experts=s.E, num_experts_per_tok=s.k, moe_intermediate_size=s.I,
+                        init_std=0.02, seed=P.configs.BASE_SEED)
+    m = P.MoE(cfg, s.k)
+    x = inp["x"].float().reshape(4, 4096, s.H).to(dev).requires_grad_(True)
+    dy = inp["dy"].float().reshape(4, 4096, s.H).to(dev)
+    flops = P.configs.gemm_flops(s)
+    out = {}
+    for name, accumulate, in_kernel in (("fresh_grads", False, False),
+                                        ("accumulating_micro_step_autograd_adds", True, False),
+                                        ("accumulating_micro_step_kernel_adds", True, True)):
+        m.accumulate_wgrad_into_grad = in_kernel
+
+        def step():
+            if not accumulate:
+                m.zero_grad(set_to_none=True)
+            x.grad = None
+            with torch.autocast("cuda", dtype=torch.bfloat16):
+                o, _ = m(x)
+            o.backward(dy)
+
+        m.zero_grad(set_to_none=True)
+        for _ in range(warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / steps
+        out[name] = {"ms_per_step": round(ms, 4), "tflops": round(flops / ms / 1e9, 1),
+                     "tokens_per_s": round(s.T / (ms * 1e-3), 1)}
+    del m
+    torch.cuda.empty_cache()
+    return {"config": 3, "workload": s.name + ", MoE module with fp32 master weights and fp32 input under bf16 "
+                                              "autocast (the reference trainer's calling convention), fp32 weight gradients",
+            "entry": "MoE.forward", **out}
 
 
 def main():
@@ -134,6 +298,8 @@ def main():
                          "profiler byte counters)")
     ap.add_argument("--cpu-fraction", type=float, default=1.0,
                     help="fraction of the tokens the CPU baseline sample processes")
+    ap.add_argument("--no-others", action="store_true",
+                    help="skip the short runs of the other benchmark configurations (field other_configs)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (one rank's share of the MoE layer, "
@@ -152,7 +318,8 @@ def main():
     torch.cuda.set_device(dev)
 
     if args.config == 5:
-        return bench_block(args, torch, P, dev)
+        print(json.dumps(bench_block(args, torch, P, dev, cpu=not args.no_cpu)), flush=True)
+        return 0
 
     inp = P.configs.make_inputs(args.config)
     s = inp["shape"]
@@ -294,35 +461,29 @@ def main():
                 "all_gemms_frac": round(flops / gemm_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4)}
 
     roofline["traffic"] = MEASURED_HBM_BYTES_PER_LAUNCH.get((args.config, roofline["kernel"]))
+    roofline["traffic_source"] = ("rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this benchmark, "
+                                  "profiles/grouped_gemm_cfg3_pmc.txt (not measured by this run)")
 
     # ---------------- CPU baseline: the oracle's per-expert loop on a bounded sample
-    cpu = None
-    if not args.no_cpu:
-        from oracle import moe_oracle as O
-        ncores = os.cpu_count() or 1
-        ncores = min(ncores, int(os.environ.get("OMP_NUM_THREADS", ncores)))
-        torch.set_num_threads(ncores)
-        cin = P.configs.make_inputs(args.config, scale_tokens=args.cpu_fraction)
-        w32 = [cin[n].float() for n in ("w1", "w3", "w2")]
-        t0 = time.perf_counter()
-        if s.rows_entry:
-            f = O.experts_rows_forward(cin["x"], cin["ids"].numpy(), *w32)
-            O.experts_rows_backward(f, cin["dy"].float(), *w32)
-            rows = cin["x"].shape[0]
-            toks = rows / s.k
-        else:
-            wr32 = cin["wr"].float()
-            f = O.moe_forward(cin["x"], wr32, *w32, s.k, bias=cin.get("bias"), logits_dtype=torch.bfloat16)
-            if s.backward:
-                O.moe_backward(f, cin["dy"].float(), wr32, *w32)
-            toks = cin["x"].shape[0]
-            rows = toks * s.k
-        dt = time.perf_counter() - t0
-        cflops = (18 if s.backward else 6) * rows * s.H * s.I
-        cpu = {"value": round(cflops / dt / 1e12, 4), "unit": "TFLOP/s", "cores": ncores, "kind": "port",
-               "sample": f"oracle per-expert loop, fp32 math on the same bf16 inputs, {int(toks)} of {s.T} tokens "
-                         f"({rows} routed rows, all {s.E} experts), one timed pass of {dt:.2f} s",
-               "tokens_per_s": round(toks / dt, 1)}
+    cpu = None if args.no_cpu else cpu_leg(P, torch, args.config, args.cpu_fraction)
+
+    # ---------------- the other benchmark configurations, briefly (the default run only)
+    others = None
+    if args.config == 3 and not args.no_others:
+        others = []
+        for cid, fraction in ((1, 1.0), (2, 1.0), (4, 1.0)):
+            rec = time_layer_config(P, torch, dev, cid, max(args.steps // 2, 5), args.warmup)
+            if not args.no_cpu:
+                rec["cpu_baseline"] = cpu_leg(P, torch, cid, fraction)
+            others.append(rec)
+        others.append(module_config3(P, torch, dev, max(args.steps // 2, 5), args.warmup))
+        blk = bench_block(args, torch, P, dev, steps=max(args.steps // 2, 5), warmup=3, cpu=not args.no_cpu)
+        others.append({"config": 5, "workload": blk["config"]["workload"], "entry": "Block.forward",
+                       "ms_per_step": blk["ms_per_step"], "tokens_per_s": blk["value"],
+                       "ms_per_step_separate_norm_and_residual": blk["ms_per_step_separate_norm_and_residual"],
+                       "moe_ms": blk["moe_ms"], "moe_share_of_block_time": blk["moe_share_of_block_time"],
+                       "moe_gemm_tflops": blk["moe_gemm_tflops"], "roofline": blk["roofline"],
+                       "cpu_baseline": blk["cpu_baseline"], "steps": blk["steps"]})
 
     line = {
         "metric": "moe_layer_fwd_bwd_tflops" if s.backward else "moe_layer_fwd_tflops",
@@ -334,7 +495,7 @@ def main():
         "tokens_per_s": round(tokens_per_s, 1),
         "ms_per_step_graph_replay": None if ms_graph is None else round(ms_graph, 4),
         "mfma_peak_frac_whole_step": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
-        "roofline": roofline, "cpu_baseline": cpu, "kernels": per_kernel,
+        "roofline": roofline, "cpu_baseline": cpu, "kernels": per_kernel, "other_configs": others,
     }
     print(json.dumps(line), flush=True)
     return 0
