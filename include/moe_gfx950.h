@@ -211,6 +211,20 @@ int moe_combine_bwd_by_token(const void* dy, int dy_dtype, const uint16_t* y, co
  * x [T,H] (bf16 or fp32), weight fp32 [H], xn bf16 [T,H], rstd fp32 [T].  H % 8 == 0, H <= 8192. */
 int moe_rmsnorm_fwd(const void* x, int x_dtype, const float* weight, float eps, int64_t T,
                     int64_t H, uint16_t* xn, float* rstd, void* stream);
+/* The same normalisation with the router behind it in one kernel (model/gpt.py:32 feeding
+ * mlp.py:100-103): besides xn and rstd it leaves the router logits bf16(xn * router_weight^T)
+ * [T,E] (what the layer returns under the reference's bf16 autocast), and the top-k ids and gates
+ * selected on them exactly as moe_router_topk_fwd would (no bias).  The normalised rows are not read a
+ * second time for the router product.  router_weight bf16 [E,H].  Supported shapes:
+ * moe_rmsnorm_router_supported(H, E, k) != 0 (H % 32 == 0, H <= 4096, E % 16 == 0, E <= 128);
+ * otherwise MOE_ERR_LIMIT and the caller runs the three separate steps.  The logits come from a
+ * different summation order than a library product's, so single bf16 logits may differ from it
+ * by one unit in the last place; ids and gates are consistent with the logits returned here. */
+int moe_rmsnorm_router_supported(int64_t H, int64_t E, int64_t k);
+int moe_rmsnorm_router_fwd(const void* x, int x_dtype, const float* weight, float eps,
+                           const uint16_t* router_weight, int64_t T, int64_t H, int64_t E, int64_t k,
+                           uint16_t* xn, float* rstd, uint16_t* logits, int32_t* ids, float* gates,
+                           void* stream);
 /* Backward of the above (autograd of norm.py:14-19), with the two gradient contributions of
  * xn summed on the way in and the residual branch's gradient added on the way out:
  *   g = d1 + d2;  xhat = x*rstd;  dx = dres + rstd * (weight*g - xhat * mean(weight*g*xhat));

@@ -225,3 +225,49 @@ def test_prenorm_moe_odd_shapes(pkg, lib, T, H, I, E, k):
     else:
         check("dx", xd.grad, dx_ref, dx_e, say=_say)
         check("d norm weight", nwd.grad, dnw_ref, dnw_e, say=_say)
+
+
+@pytest.mark.parametrize("T,H,E,k,x_dt", [
+    (1, 64, 16, 2, torch.float32), (37, 256, 32, 4, torch.float32), (300, 1024, 64, 8, torch.bfloat16),
+    (8192, 2048, 64, 8, torch.float32), (130, 4096, 128, 64, torch.bfloat16), (17, 2048, 48, 3, torch.float32),
+])
+def test_norm_router_topk_in_one_kernel(pkg, lib, T, H, E, k, x_dt):
+    """RMSNorm + router product + top-k in one kernel against the three separate steps: xn and
+    rstd are the same bits as the norm kernel's; the logits equal the library product on those
+    rows to bf16 rounding (another summation order); ids and gates are exactly what the router
+    kernel selects on the logits this kernel returned, and exactly the oracle's selection."""
+    ops = pkg.ops
+    _say(f"norm + router + top-k fused: T={T} H={H} E={E} k={k} x {x_dt}")
+    assert ops.rmsnorm_router_supported(H, E, k)
+    g = torch.Generator().manual_seed(900 + T + H + E)
+    x = (torch.randn(T, H, generator=g) * 1.4).to(x_dt).cuda()
+    w = (1.0 + 0.2 * torch.randn(H, generator=g)).cuda()
+    wr = (torch.randn(E, H, generator=g) * 0.05).to(torch.bfloat16).cuda()
+    xn0, rstd0 = ops.rmsnorm_fwd(x, w, EPS)
+    xn, rstd, logits, ids, gates = ops.rmsnorm_router_fwd(x, w, EPS, wr, k)
+    assert torch.equal(xn, xn0) and torch.equal(rstd, rstd0)
+    assert logits.dtype == torch.bfloat16 and logits.shape == (T, E)
+    want = xn.float() @ wr.float().t()
+    check("logits", logits, want.cpu(), say=_say)
+    # never further from the fp32 product than bf16 rounding plus fp32 summation-order noise
+    assert ((logits.float() - want).abs() <= want.abs() * 2.0 ** -8 + 1e-3).all()
+    ids2, gates2 = ops.router_topk(logits, k, None)
+    assert torch.equal(ids, ids2) and torch.equal(gates, gates2)
+    oid, sel = O.topk_select(logits.cpu(), k)
+    assert torch.equal(ids.cpu().reshape(T, k), torch.from_numpy(oid).to(torch.int32))
+    assert torch.allclose(gates.cpu().reshape(T, k), O.gates_from_selected(sel), atol=1e-6, rtol=1e-5)
+    again = ops.rmsnorm_router_fwd(x, w, EPS, wr, k)
+    assert all(torch.equal(a, b) for a, b in zip(again, (xn, rstd, logits, ids, gates)))  # reproducible
+
+
+def test_norm_router_unsupported_shapes_fall_back(pkg, lib):
+    ops = pkg.ops
+    assert not ops.rmsnorm_router_supported(8192, 64, 8)      # rows too long for the block's LDS tile
+    assert not ops.rmsnorm_router_supported(2048, 24, 2)      # experts not a multiple of 16
+    assert not ops.rmsnorm_router_supported(2048, 256, 8)
+    assert not ops.rmsnorm_router_supported(72, 16, 2)        # rows not a multiple of the 32-wide k-step
+    with pytest.raises(pkg.lib.MoELibError, match="MOE_ERR_LIMIT"):
+        ops.rmsnorm_router_fwd(torch.zeros(4, 72, device="cuda"), torch.ones(72, device="cuda"), EPS,
+                               torch.zeros(16, 72, dtype=torch.bfloat16, device="cuda"), 2)
+    # prenorm_moe on such a shape takes the separate kernels and still matches (covered by
+    # test_prenorm_moe_odd_shapes: H = 72 and 520, E = 3 and 6)

@@ -12,6 +12,7 @@
 // is reproducible run to run.  Both kernels are HBM-bound: each row is read once and written
 // once.
 #include "common.h"
+#include "topk_core.h"
 
 namespace {
 
@@ -78,6 +79,132 @@ __global__ __launch_bounds__(NT) void rmsnorm_fwd_kernel(const XT* __restrict__ 
         }
         store8(xn + (size_t)t * H + c * 8, o);
       }
+    }
+  }
+}
+
+// The normalisation with the router behind it (model/gpt.py:32 into model/modules/mlp.py:100-103
+// in one pass): a block normalises RB rows, keeps their bf16 form in LDS besides writing it out,
+// multiplies them with the router weight on the matrix cores (v_mfma_f32_16x16x32_bf16: rows =
+// tokens from LDS, columns = experts straight from L2, the four waves split the contraction and
+// add their partial products through LDS), rounds the logits to bf16 (what the layer returns and
+// selects on) and runs the wave-level top-k + softmax on them.  The normalised rows are not read
+// again for the router, and the logits never leave the chip before selection.
+constexpr int RB = 16;       // rows (tokens) per block
+constexpr int RMAX_EB = 8;   // 16-expert column blocks: E <= 128
+
+template <typename XT, int NV>
+__global__ __launch_bounds__(NT) void rmsnorm_router_fwd_kernel(
+    const XT* __restrict__ x, const float* __restrict__ w, float eps, int T, int H8,
+    const uint16_t* __restrict__ wr, int E, int k, uint16_t* __restrict__ xn, float* __restrict__ rstd,
+    uint16_t* __restrict__ logits, int32_t* __restrict__ ids, float* __restrict__ gates) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t rows[];  // [RB][H + 8]; later fp32 partials
+  __shared__ float red[NW];
+  __shared__ uint16_t lg16[RB * RMAX_EB * 16];
+  const int H = H8 * 8, LDT = H + 8;
+  const int lane = lane_id(), wv = threadIdx.x / MOE_WAVE;
+  const int t0 = blockIdx.x * RB;
+  Row8 wv8[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = threadIdx.x + i * NT;
+    if (c < H8) wv8[i] = load8(w + c * 8);
+  }
+  for (int rr = 0; rr < RB; ++rr) {
+    const int t = t0 + rr;
+    if (t >= T) {  // block-uniform: rows past the end are zero rows for the product
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        const int c = threadIdx.x + i * NT;
+        if (c < H8) *reinterpret_cast<u32x4*>(rows + rr * LDT + c * 8) = u32x4{0, 0, 0, 0};
+      }
+      continue;
+    }
+    Row8 xv[NV];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int c = threadIdx.x + i * NT;
+      if (c < H8) {
+        xv[i] = load8(x + (size_t)t * H + c * 8);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ss += xv[i].v[j] * xv[i].v[j];
+      }
+    }
+    ss = block_sum(ss, red);
+    const float r = rsqrtf(ss / (float)H + eps);
+    if (threadIdx.x == 0) rstd[t] = r;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int c = threadIdx.x + i * NT;
+      if (c < H8) {
+        Row8 o;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          float v = xv[i].v[j] * r;
+          if (is_bf16<XT>::value) v = bf16_to_f32(f32_to_bf16(v));  // `.to(input_dtype)`, norm.py:19
+          o.v[j] = wv8[i].v[j] * v;
+        }
+        store8(xn + (size_t)t * H + c * 8, o);
+        store8(rows + rr * LDT + c * 8, o);
+      }
+    }
+  }
+  __syncthreads();
+  // logits[m][e] = sum_h rows[m][h] * wr[e][h]: lane l holds A row l % 16 (token) and B row
+  // l % 16 of the column block (expert), 8 consecutive h at (l / 16) * 8 of the 32-wide k-step
+  const int EB = E / 16;
+  f32x4 acc[RMAX_EB];
+#pragma unroll
+  for (int nb = 0; nb < RMAX_EB; ++nb) acc[nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int l16 = lane & 15, lq = lane >> 4;
+  for (int ks = wv; ks < H / 32; ks += NW) {
+    const bf16x8 a = *reinterpret_cast<const bf16x8*>(rows + l16 * LDT + ks * 32 + lq * 8);
+#pragma unroll
+    for (int nb = 0; nb < RMAX_EB; ++nb) {
+      if (nb < EB) {
+        const bf16x8 b = *reinterpret_cast<const bf16x8*>(wr + (size_t)(nb * 16 + l16) * H + ks * 32 + lq * 8);
+        acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[nb], 0, 0, 0);
+      }
+    }
+  }
+  __syncthreads();  // every wave is done with the rows: their memory takes the partial products
+  float* part = reinterpret_cast<float*>(rows);  // [NW][RB][E]
+  // accumulator layout: lane l holds column l % 16 (expert) of rows 4 * (l / 16) .. + 3 (tokens)
+#pragma unroll
+  for (int nb = 0; nb < RMAX_EB; ++nb) {
+    if (nb < EB) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) part[(wv * RB + lq * 4 + i) * E + nb * 16 + l16] = acc[nb][i];
+    }
+  }
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < RB * E; idx += NT) {
+    float v = 0.f;
+#pragma unroll
+    for (int q = 0; q < NW; ++q) v += part[q * RB * E + idx];  // fixed order: reproducible
+    const uint16_t b = f32_to_bf16(v);
+    lg16[idx] = b;
+    const int m = idx / E;
+    if (t0 + m < T) logits[(size_t)(t0 + m) * E + (idx - m * E)] = b;
+  }
+  __syncthreads();
+  // selection: one wave per token
+  for (int m = wv; m < RB; m += NW) {
+    const int t = t0 + m;
+    if (t >= T) break;
+    uint64_t key[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int e = i * MOE_WAVE + lane;
+      key[i] = e < E ? moe_topk_key(bf16_to_f32(lg16[m * E + e]), e) : 0;
+    }
+    int my_id;
+    float my_gate;
+    moe_topk_softmax_wave<2>(key, k, lane, my_id, my_gate);
+    if (lane < k) {
+      ids[(size_t)t * k + lane] = my_id;
+      gates[(size_t)t * k + lane] = my_gate;
     }
   }
 }
@@ -231,6 +358,48 @@ extern "C" int moe_rmsnorm_fwd(const void* x, int x_dtype, const float* weight, 
   if (x_dtype == MOE_DT_BF16) return launch_fwd<uint16_t>(x, weight, eps, T, H, xn, rstd, s);
   if (x_dtype == MOE_DT_F32) return launch_fwd<float>(x, weight, eps, T, H, xn, rstd, s);
   return MOE_ERR_DTYPE;
+}
+
+extern "C" int moe_rmsnorm_router_supported(int64_t H, int64_t E, int64_t k) {
+  return (H > 0 && E > 0 && k > 0 && (H % 32) == 0 && H <= 4096 && (E % 16) == 0 && E <= 16 * RMAX_EB && k <= E &&
+          k <= MOE_MAX_TOPK)
+             ? 1 : 0;
+}
+
+extern "C" int moe_rmsnorm_router_fwd(const void* x, int x_dtype, const float* weight, float eps,
+                                      const uint16_t* router_weight, int64_t T, int64_t H, int64_t E,
+                                      int64_t k, uint16_t* xn, float* rstd, uint16_t* logits,
+                                      int32_t* ids, float* gates, void* stream) {
+  if (int rc = check_norm(T, H)) return rc;
+  if (E <= 0 || k <= 0 || k > E) return MOE_ERR_SHAPE;
+  if (!moe_rmsnorm_router_supported(H, E, k)) return MOE_ERR_LIMIT;
+  if (T == 0) return 0;
+  MOE_CHECK_PTR(x);
+  MOE_CHECK_PTR(weight);
+  MOE_CHECK_PTR(router_weight);
+  MOE_CHECK_PTR(xn);
+  if (!rstd || !logits || !ids || !gates) return MOE_ERR_NULL;
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid((unsigned)((T + RB - 1) / RB)), block(NT);
+  const size_t lds = (size_t)RB * (H + 8) * 2 > (size_t)NW * RB * E * 4 ? (size_t)RB * (H + 8) * 2 : (size_t)NW * RB * E * 4;
+#define MOE_NORM_ROUTER(XT, NV)                                                                          \
+  do {                                                                                                   \
+    auto kern = rmsnorm_router_fwd_kernel<XT, NV>;                                                       \
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+    if (e != hipSuccess) return (int)e;                                                                  \
+    hipLaunchKernelGGL(kern, grid, block, lds, s, (const XT*)x, weight, eps, (int)T, (int)(H / 8),       \
+                       router_weight, (int)E, (int)k, xn, rstd, logits, ids, gates);                     \
+  } while (0)
+  const int nv = pick_nv(H);
+  if (x_dtype == MOE_DT_BF16) {
+    if (nv == 1) MOE_NORM_ROUTER(uint16_t, 1); else MOE_NORM_ROUTER(uint16_t, 2);
+  } else if (x_dtype == MOE_DT_F32) {
+    if (nv == 1) MOE_NORM_ROUTER(float, 1); else MOE_NORM_ROUTER(float, 2);
+  } else {
+    return MOE_ERR_DTYPE;
+  }
+#undef MOE_NORM_ROUTER
+  return moe_launch_status();
 }
 
 extern "C" int64_t moe_rmsnorm_bwd_workspace_bytes(int64_t T, int64_t H) {

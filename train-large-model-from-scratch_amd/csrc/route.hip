@@ -5,37 +5,10 @@
 // max-reduction over 64-bit keys, and the softmax over the k winners is a wave reduction.
 // HBM-bound: reads T*E logits, writes T*k ids and gates.
 #include "common.h"
+#include "topk_core.h"
 
 namespace {
 
-__device__ __forceinline__ uint32_t orderable(float v) {
-  v += 0.0f;  // -0.0 -> +0.0 so that the two compare equal, as they do for torch.topk
-  uint32_t u = __builtin_bit_cast(uint32_t, v);
-  return u ^ ((u >> 31) ? 0xffffffffu : 0x80000000u);
-}
-__device__ __forceinline__ float from_orderable(uint32_t u) {
-  u ^= ((u >> 31) ? 0x80000000u : 0xffffffffu);
-  return __builtin_bit_cast(float, u);
-}
-
-__device__ __forceinline__ uint64_t wave_max_u64(uint64_t v) {
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) {
-    uint32_t lo = __shfl_xor((uint32_t)v, off, MOE_WAVE);
-    uint32_t hi = __shfl_xor((uint32_t)(v >> 32), off, MOE_WAVE);
-    uint64_t o = ((uint64_t)hi << 32) | lo;
-    v = o > v ? o : v;
-  }
-  return v;
-}
-__device__ __forceinline__ float wave_sum_f32(float v) {
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, MOE_WAVE);
-  return v;
-}
-
-// key = (orderable(logit) << 32) | (0xffffffff - expert): the maximum key is the largest
-// logit and, among equal logits, the smallest expert index.  0 marks "taken / absent".
 template <int VPL, typename LT>
 __global__ __launch_bounds__(256) void router_topk_fwd_kernel(const LT* __restrict__ logits,
                                                              const float* __restrict__ bias,
@@ -55,31 +28,15 @@ __global__ __launch_bounds__(256) void router_topk_fwd_kernel(const LT* __restri
       if constexpr (sizeof(LT) == 2) v = bf16_to_f32(((const uint16_t*)logits)[(size_t)t * E + e]);
       else v = ((const float*)logits)[(size_t)t * E + e];
       if (bias) v += bias[e];
-      key[i] = ((uint64_t)orderable(v) << 32) | (uint64_t)(0xffffffffu - (uint32_t)e);
+      key[i] = moe_topk_key(v, e);
     }
   }
-  int my_id = 0;
-  float my_val = 0.f;
-  for (int j = 0; j < k; ++j) {
-    uint64_t best = key[0];
-#pragma unroll
-    for (int i = 1; i < VPL; ++i) best = key[i] > best ? key[i] : best;
-    best = wave_max_u64(best);
-    const uint32_t e = 0xffffffffu - (uint32_t)best;
-#pragma unroll
-    for (int i = 0; i < VPL; ++i)
-      if ((int)e == i * MOE_WAVE + lane) key[i] = 0;
-    if (lane == j) {
-      my_id = (int)e;
-      my_val = from_orderable((uint32_t)(best >> 32));
-    }
-  }
-  const float vmax = __shfl(my_val, 0, MOE_WAVE);
-  const float p = lane < k ? expf(my_val - vmax) : 0.f;
-  const float s = wave_sum_f32(p);
+  int my_id;
+  float my_gate;
+  moe_topk_softmax_wave<VPL>(key, k, lane, my_id, my_gate);
   if (lane < k) {
     ids[(size_t)t * k + lane] = my_id;
-    gates[(size_t)t * k + lane] = p / s;
+    gates[(size_t)t * k + lane] = my_gate;
   }
 }
 
@@ -99,7 +56,7 @@ __global__ __launch_bounds__(256) void router_topk_bwd_kernel(const float* __res
     dg = dgates[(size_t)t * k + lane];
     id = ids[(size_t)t * k + lane];
   }
-  const float s = wave_sum_f32(g * dg);
+  const float s = moe_wave_sum_f32(g * dg);
   const float dsel = g * (dg - s);
   float val[VPL];
 #pragma unroll

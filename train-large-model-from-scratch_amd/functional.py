@@ -258,15 +258,21 @@ class _PreNormMoE(torch.autograd.Function):
         w1b, w3b, w2b = (sh if sh is not None else ops.cast_bf16(w.contiguous())
                          for w, sh in zip((w1, w3, w2), shadows))
         wrb = wr.detach().to(torch.bfloat16)
-        if norm_w is not None:
+        if norm_w is not None and bias is None and T > 0 and ops.rmsnorm_router_supported(H, E, k):
+            # norm, router product and selection in one kernel: the normalised rows are not read
+            # a second time for the router, the logits are selected on before they leave the chip
             nw = norm_w.detach().float().contiguous()
-            xn, rstd = ops.rmsnorm_fwd(x, nw, eps)
+            xn, rstd, logits, ids, gates = ops.rmsnorm_router_fwd(x, nw, eps, wrb.contiguous(), k)
         else:
-            nw = rstd = None
-            xn = ops.cast_bf16(x)
-        with torch.autocast("cuda", enabled=False):
-            logits = xn @ wrb.t()
-        ids, gates = ops.router_topk(logits, k, bias)
+            if norm_w is not None:
+                nw = norm_w.detach().float().contiguous()
+                xn, rstd = ops.rmsnorm_fwd(x, nw, eps)
+            else:
+                nw = rstd = None
+                xn = ops.cast_bf16(x)
+            with torch.autocast("cuda", enabled=False):
+                logits = xn @ wrb.t()
+            ids, gates = ops.router_topk(logits, k, bias)
         counts, offs, pos_to_row, row_to_pos = ops.histogram_scan(ids, E)
         xp = ops.permute_fwd(xn, pos_to_row, k, row_to_pos)
         train = any(ctx.needs_input_grad)

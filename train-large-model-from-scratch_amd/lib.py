@@ -37,6 +37,9 @@ SIGNATURES = {
     "moe_combine_bwd": (_int, [_vp, _int, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _vp]),
     "moe_combine_fwd_residual": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _int, _vp]),
     "moe_rmsnorm_fwd": (_int, [_vp, _int, _vp, ctypes.c_float, _i64, _i64, _vp, _vp, _vp]),
+    "moe_rmsnorm_router_supported": (_int, [_i64, _i64, _i64]),
+    "moe_rmsnorm_router_fwd": (_int, [_vp, _int, _vp, ctypes.c_float, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _vp,
+                                      _vp, _vp, _vp]),
     "moe_rmsnorm_bwd_workspace_bytes": (_i64, [_i64, _i64]),
     "moe_rmsnorm_bwd": (_int, [_vp, _int, _vp, _vp, _vp, _int, _vp, _vp, _i64, _i64, _vp, _vp, _vp,
                                _i64, _vp]),

@@ -202,6 +202,27 @@ def rmsnorm_fwd(x: torch.Tensor, weight: torch.Tensor, eps: float):
     return xn, rstd
 
 
+def rmsnorm_router_supported(H: int, E: int, k: int) -> bool:
+    return bool(_lib.load().cdll.moe_rmsnorm_router_supported(H, E, k))
+
+
+def rmsnorm_router_fwd(x: torch.Tensor, weight: torch.Tensor, eps: float, router_weight: torch.Tensor, k: int):
+    """RMSNorm, router product and top-k in one kernel: x [T,H], norm weight fp32 [H], router
+    weight bf16 [E,H] -> xn bf16 [T,H], rstd fp32 [T], logits bf16 [T,E], ids int32 [T*k],
+    gates fp32 [T*k]."""
+    T, H = x.shape
+    E = router_weight.shape[0]
+    dev = x.device
+    xn = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+    rstd = torch.empty(T, dtype=torch.float32, device=dev)
+    logits = torch.empty(T, E, dtype=torch.bfloat16, device=dev)
+    ids = torch.empty(T * k, dtype=torch.int32, device=dev)
+    gates = torch.empty(T * k, dtype=torch.float32, device=dev)
+    _lib.load().call("moe_rmsnorm_router_fwd", _p(x), _dt(x), _p(weight), float(eps), _p(router_weight), T, H, E, k,
+                     _p(xn), _p(rstd), _p(logits), _p(ids), _p(gates), _stream())
+    return xn, rstd, logits, ids, gates
+
+
 def rmsnorm_bwd(x, weight, rstd, d1, d2=None, dres=None):
     """-> dx [T,H] (dtype of x), dweight fp32 [H]; see include/moe_gfx950.h."""
     T, H = x.shape
