@@ -450,6 +450,20 @@ def main():
                 rec.update(bound="hbm", achieved=round(by / kms / 1e6, 1), unit="GB/s",
                            frac=round(by / kms / 1e6 / HBM_PEAK_GBS, 4))
             per_kernel.append(rec)
+        # what the vendor's dense GEMM library reaches on this part on problems of the same size
+        # with none of the layer's structure (one weight for all rows, no ragged groups, no fused
+        # epilogue, one output): the practical ceiling the grouped kernels are measured against
+        lib_ref = {}
+        if True:
+            wd = torch.randn(2 * I, H, device=dev).to(bf) * 0.02
+            wdn = torch.randn(H, I, device=dev).to(bf) * 0.02
+            t_gu = _event_time_ms(torch, lambda: torch.mm(xp, wd.t()), 10, 3)
+            t_dn = _event_time_ms(torch, lambda: torch.mm(act, wdn.t()), 10, 3)
+            lib_ref = {"what": "torch.mm (hipBLASLt) on dense problems of the gate/up and down sizes: "
+                               "[R,H]x[H,2I] and [R,I]x[I,H], bf16, same random data scale",
+                       "gateup_size_tflops": round(4 * RHI / t_gu / 1e9, 1), "down_size_tflops": round(2 * RHI / t_dn / 1e9, 1),
+                       "gateup_size_frac_of_peak": round(4 * RHI / t_gu / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4)}
+            del wd, wdn
     gemms = [r for r in per_kernel if r["bound"] == "mfma"]
     if not s.backward:
         gemms = gemms[:2]
@@ -495,7 +509,8 @@ def main():
         "tokens_per_s": round(tokens_per_s, 1),
         "ms_per_step_graph_replay": None if ms_graph is None else round(ms_graph, 4),
         "mfma_peak_frac_whole_step": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
-        "roofline": roofline, "cpu_baseline": cpu, "kernels": per_kernel, "other_configs": others,
+        "roofline": roofline, "cpu_baseline": cpu, "kernels": per_kernel, "library_dense_reference": lib_ref,
+        "other_configs": others,
     }
     print(json.dumps(line), flush=True)
     return 0
