@@ -28,12 +28,12 @@ HBM_PEAK_GBS = 8000.0
 # are in profiles/grouped_gemm_cfg3_pmc.txt.  bench.py cannot run the profiler on itself, so
 # the figures are carried here and refreshed whenever that profile is.
 MEASURED_HBM_BYTES_PER_LAUNCH = {
-    (3, "gemm_gateup_swiglu_fwd"): 4.010e9,
-    (3, "gemm_down_fwd"): 1.830e9,
-    (3, "gemm_dgrad_down_swiglu_bwd"): 2.452e9,
-    (3, "gemm_dgrad_gateup"): 3.791e9,
+    (3, "gemm_gateup_swiglu_fwd"): 3.996e9,
+    (3, "gemm_down_fwd"): 1.816e9,
+    (3, "gemm_dgrad_down_swiglu_bwd"): 2.458e9,
+    (3, "gemm_dgrad_gateup"): 3.803e9,
     (3, "gemm_wgrad_down"): 1.074e9,
-    (3, "gemm_wgrad_gate_or_up"): 1.074e9,
+    (3, "gemm_wgrad_gate_and_up_pair"): 2.19e9,   # from the average over both weight-gradient launches
 }
 
 
@@ -412,8 +412,16 @@ def main():
         dyy = dy if dy is not None else torch.randn_like(xd)
         dyp, _ = ops.combine_bwd(dyy, None, gates, p2r, kk, r2p)
         routed = gates is not None  # the gate gradients' block sums ride in the dgrad-down kernel
-        dg, du = ops.gemm_dgrad_down(dyp, w2, g, u, offs, dgate_blocks=routed)[:2]
-        dxp = ops.gemm_dgrad_gateup(dg, du, w1, w3, offs)
+        # (dg and du side by side in one buffer, as the backward pass keeps them when I % 256 == 0:
+        # their two weight gradients are then one launch)
+        packed = s.I % 256 == 0
+        if packed:
+            dgu = ops.gemm_dgrad_down_packed(dyp, w2, g, u, offs, dgate_blocks=routed)[0]
+            dxp = ops.gemm_dgrad_gateup_packed(dgu, w1, w3, offs)
+            dg = dgu[:, :s.I].contiguous()
+        else:
+            dg, du = ops.gemm_dgrad_down(dyp, w2, g, u, offs, dgate_blocks=routed)[:2]
+            dxp = ops.gemm_dgrad_gateup(dg, du, w1, w3, offs)
         bf = torch.bfloat16
         a = 2  # bytes per bf16 element
         T, R, H, I, E = xd.shape[0], s.R, s.H, s.I, s.E
@@ -421,11 +429,15 @@ def main():
             # name, callable, algorithmic flops, algorithmic bytes, launches per step
             ("gemm_gateup_swiglu_fwd", lambda: ops.gemm_gateup(xp, w1, w3, offs, True), 4 * RHI, 0, 1),
             ("gemm_down_fwd", lambda: ops.gemm_down(act, w2, offs), 2 * RHI, 0, 1),
-            ("gemm_dgrad_down_swiglu_bwd", lambda: ops.gemm_dgrad_down(dyp, w2, g, u, offs, dgate_blocks=routed),
-             2 * RHI, 0, 1),
-            ("gemm_dgrad_gateup", lambda: ops.gemm_dgrad_gateup(dg, du, w1, w3, offs), 4 * RHI, 0, 1),
+            ("gemm_dgrad_down_swiglu_bwd",
+             (lambda: ops.gemm_dgrad_down_packed(dyp, w2, g, u, offs, dgate_blocks=routed)) if packed else
+             (lambda: ops.gemm_dgrad_down(dyp, w2, g, u, offs, dgate_blocks=routed)), 2 * RHI, 0, 1),
+            ("gemm_dgrad_gateup",
+             (lambda: ops.gemm_dgrad_gateup_packed(dgu, w1, w3, offs)) if packed else
+             (lambda: ops.gemm_dgrad_gateup(dg, du, w1, w3, offs)), 4 * RHI, 0, 1),
             ("gemm_wgrad_down", lambda: ops.gemm_wgrad(dyp, act, offs, E, bf), 2 * RHI, 0, 1),
-            ("gemm_wgrad_gate_or_up", lambda: ops.gemm_wgrad(dg, xp, offs, E, bf), 2 * RHI, 0, 2),
+            (("gemm_wgrad_gate_and_up_pair", lambda: ops.gemm_wgrad_pair(dgu, xp, offs, E, bf), 4 * RHI, 0, 1) if packed
+             else ("gemm_wgrad_gate_or_up", lambda: ops.gemm_wgrad(dg, xp, offs, E, bf), 2 * RHI, 0, 2)),
             ("permute_fwd", lambda: ops.permute_fwd(xd, p2r, kk, r2p), 0, T * H * a + R * H * a + R * 4, 1),
             ("combine_fwd", lambda: ops.combine_fwd(y, gates, r2p, T, kk, xd.dtype), 0,
              R * H * a + R * 8 + T * H * a, 1),

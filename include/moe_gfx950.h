@@ -170,6 +170,24 @@ int moe_gemm_wgrad(const uint16_t* a, const uint16_t* b, const int32_t* offs, in
                    int64_t R, int64_t M, int64_t N, void* dw, int dw_dtype, int accumulate,
                    void* stream);
 
+/* The gate and up halves of the backward in one buffer.  dgu bf16 [R, 2I] holds each row's dg and
+ * du side by side ([dg row | du row]); then dgu^T * xp is ONE grouped weight-gradient product
+ * whose result rows 0..I-1 are dW1 and I..2I-1 are dW3: one launch instead of two, xp read once
+ * per column tile (autograd of mlp.py:154-155 w.r.t. both weights).  The three calls compute what
+ * moe_gemm_dgrad_down_swiglu_bwd[_dgate] (dgate_part may be NULL), moe_gemm_dgrad_gateup and two
+ * moe_gemm_wgrad calls compute, bit for bit.  moe_gemm_wgrad_pair needs I % 256 == 0
+ * (MOE_ERR_SHAPE otherwise: take the separate calls on dgu's two column halves). */
+int moe_gemm_dgrad_down_swiglu_bwd_packed(const uint16_t* dyp, const uint16_t* w2, const uint16_t* g,
+                                          const uint16_t* u, const int32_t* offs, int64_t E, int64_t R,
+                                          int64_t H, int64_t I, uint16_t* dgu, float* dgate_part,
+                                          void* stream);
+int moe_gemm_dgrad_gateup_packed(const uint16_t* dgu, const uint16_t* w1, const uint16_t* w3,
+                                 const int32_t* offs, int64_t E, int64_t R, int64_t H, int64_t I,
+                                 uint16_t* dxp, void* stream);
+int moe_gemm_wgrad_pair(const uint16_t* dgu, const uint16_t* xp, const int32_t* offs, int64_t E,
+                        int64_t R, int64_t I, int64_t H, void* dw1, void* dw3, int dw_dtype,
+                        int accumulate, void* stream);
+
 /* Row segments for a weight gradient whose output has too few tiles to fill the chip: every
  * expert's row range is cut into S equal parts, seg[e*S+s] = offs[e] + (offs[e+1]-offs[e])*s/S,
  * seg[E*S] = offs[E].  moe_gemm_wgrad over seg with E*S "experts" and fp32 output gives S

@@ -367,6 +367,40 @@ def test_gate_gradients_from_the_dgrad_down_kernel(ops, R, H, I, E, empty):
     assert torch.equal(again, dgates)  # reproducible
 
 
+@pytest.mark.parametrize("R,H,I,E,empty", [(1000, 256, 256, 5, ()), (3000, 520, 512, 7, (2, 5)), (8192, 1024, 1024, 8, ()),
+                                           (130, 64, 256, 16, (0, 15))])
+def test_packed_row_gradients_and_paired_weight_gradients(pkg, ops, R, H, I, E, empty):
+    """dg and du side by side in one buffer and both their weight gradients from one launch:
+    the same bits as the separate kernels (same tiles, same order of additions), with fp32 and
+    bf16 results, with accumulation, and with the gate gradients' block sums."""
+    _say("packed dg|du and paired wgrad", R, H, I, E, empty)
+    xp, w1, w3, w2, starts = _gemm_case(R, H, I, E, seed=R + I + 1, empty=empty)
+    offs = torch.from_numpy(starts).cuda()
+    xp, w1, w3, w2 = xp.cuda(), w1.cuda(), w3.cuda(), w2.cuda()
+    dyp = torch.randn(R, H, generator=torch.Generator().manual_seed(2)).to(torch.bfloat16).cuda()
+    g, u, act = ops.gemm_gateup(xp, w1, w3, offs, save_gu=True)
+    dg, du, part = ops.gemm_dgrad_down(dyp, w2, g, u, offs, dgate_blocks=True)
+    dgu, part2 = ops.gemm_dgrad_down_packed(dyp, w2, g, u, offs, dgate_blocks=True)
+    assert dgu.shape == (R, 2 * I)
+    assert torch.equal(dgu[:, :I], dg) and torch.equal(dgu[:, I:], du) and torch.equal(part2, part)
+    dgu3, none = ops.gemm_dgrad_down_packed(dyp, w2, g, u, offs)
+    assert none is None and torch.equal(dgu3, dgu)
+    assert torch.equal(ops.gemm_dgrad_gateup_packed(dgu, w1, w3, offs), ops.gemm_dgrad_gateup(dg, du, w1, w3, offs))
+    for dt in (torch.float32, torch.bfloat16):
+        a1, a3 = ops.gemm_wgrad_pair(dgu, xp, offs, E, dt)
+        b1, b3 = ops.gemm_wgrad(dg, xp, offs, E, dt), ops.gemm_wgrad(du, xp, offs, E, dt)
+        assert torch.equal(a1, b1) and torch.equal(a3, b3)
+        ops.gemm_wgrad_pair(dgu, xp, offs, E, dt, out1=a1, out3=a3)        # accumulate into the results
+        ops.gemm_wgrad(dg, xp, offs, E, dt, out=b1)
+        ops.gemm_wgrad(du, xp, offs, E, dt, out=b3)
+        assert torch.equal(a1, b1) and torch.equal(a3, b3)
+        for e in empty:
+            assert not a1[e].any() and not a3[e].any()
+    if I == 256:  # a width whose 256-row tiles would straddle the halves is refused
+        with pytest.raises(pkg.lib.MoELibError, match="MOE_ERR_SHAPE"):
+            ops.gemm_wgrad_pair(dgu[:, :2 * 136].contiguous(), xp, offs, E, torch.float32)
+
+
 def test_grouped_gemms_on_buffers_beyond_4_gib(ops):
     """Row buffers larger than 4 GiB, one expert owning more than 4 GiB of them: the rows on
     both sides of the 2^32-byte mark (row 2^20 at 4096 bytes per row) and the last rows must come

@@ -53,6 +53,9 @@ struct GemmArgs {
   int n_tiles;  // tiles along N
   int m_slots;  // row-tile slots (ragged modes) or tiles along M (WGRAD)
   int accumulate;
+  int ld_a;     // row stride of A0/A1 in elements when it is not the contraction length (0: K)
+  int ld_c;     // row stride of the outputs C0/C1 in elements when it is not N (0: N)
+  int m_split;  // WGRAD: rows m >= m_split of an expert's result go to C1 (as its rows m - m_split); 0: all to C0
 };
 
 template <int BM_, int BN_, int BK_, int WM_, int WN_, int NSET_>
@@ -346,7 +349,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WAVES_PER_SIMD) void grouped_gemm_ker
   int lda, ldb;
   if constexpr (MODE == GATEUP || MODE == DOWN) lda = ldb = p.K;
   else if constexpr (MODE == WGRAD) { lda = p.M; ldb = p.N; }
-  else { lda = p.K; ldb = p.N; }
+  else { lda = p.ld_a ? p.ld_a : p.K; ldb = p.N; }
 
   // Fills `t` for tile slot `logical`; false when the slot lies past the last real tile.
   // Every lane computes the same thing from the same LDS words / scalar loads.
@@ -611,7 +614,8 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WAVES_PER_SIMD) void grouped_gemm_ker
                     ? reinterpret_cast<char*>(wv < HALF_WAVES ? sA + StA::LDS_ELEMS : sB + StB::LDS_ELEMS) +
                           (wv % HALF_WAVES) * (NSTRIP * SBYTES)
                     : reinterpret_cast<char*>(smem) + wv * (NSTRIP * SBYTES);
-  const int ldc = p.N;
+  const int ldc = p.ld_c ? p.ld_c : p.N;  // outputs
+  const int ldx = p.N;                    // epilogue inputs (g, u)
   auto acc_ptr = [&](int plane, int j, int q) {  // 4 consecutive columns in accumulator layout
     return strip + plane * SBYTES + l32 * SSTRIDE + (j * 32 + 8 * q + 4 * lh) * OSZ;
   };
@@ -631,7 +635,23 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WAVES_PER_SIMD) void grouped_gemm_ker
   // `halfway` runs once, after the second of the FM strips
   auto epilogue = [&](const Tile& t, auto&& halfway) {
     const int col_w0 = t.n0 + wn * WTNC;  // first output column of the wave
-    const int row_lim = (MODE == WGRAD) ? p.M : t.row_end;
+    char* C0 = (char*)p.C0;
+    int m_shift = 0;  // WGRAD with two results: the rows of the second one start at m_split
+    int m_lim = p.M;
+    if constexpr (MODE == WGRAD) {
+      if (p.m_split > 0) {
+        if (t.m0 >= p.m_split) {
+          C0 = (char*)p.C1 + (long long)t.e * (p.M - p.m_split) * p.N * OSZ;
+          m_shift = p.m_split;
+        } else {
+          C0 += (long long)t.e * p.m_split * p.N * OSZ;
+          m_lim = p.m_split;
+        }
+      } else {
+        C0 += (long long)t.e * p.M * p.N * OSZ;
+      }
+    }
+    const int row_lim = (MODE == WGRAD) ? m_lim : t.row_end;
     // row-wise pass over a strip: lane handles chunk (lane % CPRO) of row it*RPI + lane/CPRO
     auto store_rows = [&](int plane, int i, char* gbase /* element (0,0) of the output */) {
       const int rbase = (MODE == WGRAD ? t.m0 : t.row0) + wm * WTM + i * 32;
@@ -641,7 +661,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WAVES_PER_SIMD) void grouped_gemm_ker
         const u32x4 v = *reinterpret_cast<const u32x4*>(strip + plane * SBYTES + rr * SSTRIDE + ch * 16);
         const int r = rbase + rr, c = col_w0 + ch * (16 / OSZ);
         if (r < row_lim && c < p.N) {
-          u32x4* dst = reinterpret_cast<u32x4*>(gbase + ((long long)r * ldc + c) * OSZ);
+          u32x4* dst = reinterpret_cast<u32x4*>(gbase + ((long long)(r - m_shift) * ldc + c) * OSZ);
           if (MODE == WGRAD && p.accumulate) {
             const u32x4 o = *dst;
             if constexpr (OSZ == 4) {
@@ -674,8 +694,8 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WAVES_PER_SIMD) void grouped_gemm_ker
         rr_.g[it] = u32x4{0, 0, 0, 0};
         rr_.u[it] = u32x4{0, 0, 0, 0};
         if (r < row_lim && c < p.N) {
-          rr_.g[it] = *reinterpret_cast<const u32x4*>((const char*)p.X0 + ((long long)r * ldc + c) * OSZ);
-          rr_.u[it] = *reinterpret_cast<const u32x4*>((const char*)p.X1 + ((long long)r * ldc + c) * OSZ);
+          rr_.g[it] = *reinterpret_cast<const u32x4*>((const char*)p.X0 + ((long long)r * ldx + c) * OSZ);
+          rr_.u[it] = *reinterpret_cast<const u32x4*>((const char*)p.X1 + ((long long)r * ldx + c) * OSZ);
         }
       }
     };
@@ -689,8 +709,6 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WAVES_PER_SIMD) void grouped_gemm_ker
     };
     RowRegs rows_in;
     if constexpr (MODE == DGRAD_DOWN) request_rows(0, rows_in);
-    char* C0 = (char*)p.C0;
-    if constexpr (MODE == WGRAD) C0 += (long long)t.e * p.M * p.N * OSZ;
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
       if constexpr (MODE == GATEUP) {
@@ -976,7 +994,7 @@ extern "C" int64_t moe_dgate_blocks(int64_t I) {
 
 static int dgrad_down_impl(const uint16_t* dyp, const uint16_t* w2, const uint16_t* g, const uint16_t* u,
                            const int32_t* offs, int64_t E, int64_t R, int64_t H, int64_t I,
-                           uint16_t* dg, uint16_t* du, float* dgate_part, void* stream) {
+                           uint16_t* dg, uint16_t* du, float* dgate_part, void* stream, int64_t ld_out = 0) {
   if (int rc = check_common(offs, E, R, H, I)) return rc;
   if (R == 0) return 0;
   MOE_CHECK_PTR(dyp); MOE_CHECK_PTR(w2); MOE_CHECK_PTR(g); MOE_CHECK_PTR(u);
@@ -985,7 +1003,7 @@ static int dgrad_down_impl(const uint16_t* dyp, const uint16_t* w2, const uint16
   GemmArgs a{};
   a.C2 = dgate_part;
   a.A0 = dyp; a.B0 = w2; a.X0 = g; a.X1 = u; a.C0 = dg; a.C1 = du; a.offs = offs;
-  a.E = (int)E; a.R = (int)R; a.N = (int)I; a.K = (int)H;
+  a.E = (int)E; a.R = (int)R; a.N = (int)I; a.K = (int)H; a.ld_c = (int)ld_out;
   a.n_tiles = (int)((I + Cfg::BN - 1) / Cfg::BN);
   a.m_slots = row_slots<Cfg>(R, E);
   return launch<DGRAD_DOWN, Cfg, uint16_t>(a, (long long)a.n_tiles * a.m_slots, (hipStream_t)stream);
@@ -1007,19 +1025,64 @@ extern "C" int moe_gemm_dgrad_down_swiglu_bwd_dgate(const uint16_t* dyp, const u
   return dgrad_down_impl(dyp, w2, g, u, offs, E, R, H, I, dg, du, dgate_part, stream);
 }
 
-extern "C" int moe_gemm_dgrad_gateup(const uint16_t* dg, const uint16_t* du, const uint16_t* w1,
-                                     const uint16_t* w3, const int32_t* offs, int64_t E, int64_t R,
-                                     int64_t H, int64_t I, uint16_t* dxp, void* stream) {
+// The two row gradients side by side in one buffer: dgu [R, 2I], row = [dg row | du row].  The
+// weight gradients of the gate and up stacks then are ONE grouped product, dgu^T * xp, whose
+// result rows 0..I-1 are dW1 and I..2I-1 dW3 (moe_gemm_wgrad_pair).
+extern "C" int moe_gemm_dgrad_down_swiglu_bwd_packed(const uint16_t* dyp, const uint16_t* w2,
+                                                     const uint16_t* g, const uint16_t* u,
+                                                     const int32_t* offs, int64_t E, int64_t R,
+                                                     int64_t H, int64_t I, uint16_t* dgu,
+                                                     float* dgate_part, void* stream) {
+  if (R > 0 && !dgu) return MOE_ERR_NULL;
+  return dgrad_down_impl(dyp, w2, g, u, offs, E, R, H, I, dgu, dgu ? dgu + I : nullptr, dgate_part, stream, 2 * I);
+}
+
+static int dgrad_gateup_impl(const uint16_t* dg, const uint16_t* du, int64_t ld_in, const uint16_t* w1,
+                             const uint16_t* w3, const int32_t* offs, int64_t E, int64_t R, int64_t H,
+                             int64_t I, uint16_t* dxp, void* stream) {
   if (int rc = check_common(offs, E, R, H, I)) return rc;
   if (R == 0) return 0;
   MOE_CHECK_PTR(dg); MOE_CHECK_PTR(du); MOE_CHECK_PTR(w1); MOE_CHECK_PTR(w3); MOE_CHECK_PTR(dxp);
   using Cfg = CfgMain;
   GemmArgs a{};
-  a.A0 = dg; a.A1 = du; a.B0 = w1; a.B1 = w3; a.C0 = dxp; a.offs = offs;
+  a.A0 = dg; a.A1 = du; a.B0 = w1; a.B1 = w3; a.C0 = dxp; a.offs = offs; a.ld_a = (int)ld_in;
   a.E = (int)E; a.R = (int)R; a.N = (int)H; a.K = (int)I;
   a.n_tiles = (int)((H + Cfg::BN - 1) / Cfg::BN);
   a.m_slots = row_slots<Cfg>(R, E);
   return launch<DGRAD_GATEUP, Cfg, uint16_t>(a, (long long)a.n_tiles * a.m_slots, (hipStream_t)stream);
+}
+
+extern "C" int moe_gemm_dgrad_gateup_packed(const uint16_t* dgu, const uint16_t* w1, const uint16_t* w3,
+                                            const int32_t* offs, int64_t E, int64_t R, int64_t H,
+                                            int64_t I, uint16_t* dxp, void* stream) {
+  if (R > 0 && !dgu) return MOE_ERR_NULL;
+  return dgrad_gateup_impl(dgu, dgu ? dgu + I : nullptr, 2 * I, w1, w3, offs, E, R, H, I, dxp, stream);
+}
+
+extern "C" int moe_gemm_wgrad_pair(const uint16_t* dgu, const uint16_t* xp, const int32_t* offs, int64_t E,
+                                   int64_t R, int64_t I, int64_t H, void* dw1, void* dw3, int dw_dtype,
+                                   int accumulate, void* stream) {
+  if (int rc = check_common(offs, E, R, 2 * I, H)) return rc;
+  // a 256-row tile of the stacked result must not straddle the two halves
+  if ((I % CfgMain::BM) != 0) return MOE_ERR_SHAPE;
+  MOE_CHECK_PTR(dw1); MOE_CHECK_PTR(dw3);
+  if (R > 0) { MOE_CHECK_PTR(dgu); MOE_CHECK_PTR(xp); }
+  if (dw_dtype != MOE_DT_BF16 && dw_dtype != MOE_DT_F32) return MOE_ERR_DTYPE;
+  using Cfg = CfgMain;
+  GemmArgs a{};
+  a.A0 = dgu; a.B0 = xp; a.C0 = dw1; a.C1 = dw3; a.offs = offs; a.m_split = (int)I;
+  a.E = (int)E; a.R = (int)R; a.M = (int)(2 * I); a.N = (int)H; a.accumulate = accumulate;
+  a.n_tiles = (int)((H + Cfg::BN - 1) / Cfg::BN);
+  a.m_slots = (int)((2 * I + Cfg::BM - 1) / Cfg::BM);
+  const long long nblocks = (long long)a.n_tiles * a.m_slots * E;
+  if (dw_dtype == MOE_DT_F32) return launch<WGRAD, Cfg, float>(a, nblocks, (hipStream_t)stream);
+  return launch<WGRAD, Cfg, uint16_t>(a, nblocks, (hipStream_t)stream);
+}
+
+extern "C" int moe_gemm_dgrad_gateup(const uint16_t* dg, const uint16_t* du, const uint16_t* w1,
+                                     const uint16_t* w3, const int32_t* offs, int64_t E, int64_t R,
+                                     int64_t H, int64_t I, uint16_t* dxp, void* stream) {
+  return dgrad_gateup_impl(dg, du, 0, w1, w3, offs, E, R, H, I, dxp, stream);
 }
 
 extern "C" int moe_gemm_wgrad(const uint16_t* a_, const uint16_t* b_, const int32_t* offs, int64_t E,

@@ -150,14 +150,54 @@ def _wgrad(a, b, offs, E, wdtype, needed, param):
     return _gemm_wgrad(a, b, offs, E, wdtype)  # a .grad the kernel cannot add to: autograd sums
 
 
+def _grad_slot_ok(param, shape, device):
+    held = param.grad
+    return held is None or (held.dtype in (torch.float32, torch.bfloat16) and held.is_contiguous()
+                            and tuple(held.shape) == tuple(shape) and held.device == device)
+
+
+def _pair_ok(E, I, H, need_w, into, device):
+    """Whether the gate and up weight gradients can come out of one launch on the side-by-side
+    [dg | du] buffer: both wanted, 256-row tiles of the stacked result do not straddle the halves,
+    the launch fills the chip without a row split, and (when the kernel is to add into `.grad`)
+    both slots are in the same state."""
+    if not (need_w[0] and need_w[1]) or I % _WGRAD_TILE != 0 or _wgrad_split(E, I, H, device) != 1:
+        return False
+    p1, p3 = into[0], into[1]
+    if p1 is None and p3 is None:
+        return True
+    if p1 is None or p3 is None:
+        return False
+    shape = (E, I, H)
+    if not (_grad_slot_ok(p1, shape, device) and _grad_slot_ok(p3, shape, device)):
+        return False
+    g1, g3 = p1.grad, p3.grad
+    return (g1 is None) == (g3 is None) and (g1 is None or g1.dtype == g3.dtype) and p1.dtype == p3.dtype
+
+
 def _expert_backward(dyp, xp, g, u, act, w1b, w3b, w2b, offs, wdtype, need_w=(True, True, True),
                      into=None, gate_blocks=False):
     """Shared backward of the expert FFN over expert-contiguous rows.  `need_w` and `into`
     are per stack in the order gate, up, down.  With `gate_blocks` the fifth result holds the
     per-row block sums of <dact, act> (the gate gradients are made from them), else None."""
-    E = w1b.shape[0]
+    E, I, H = w1b.shape
     into = into or (None, None, None)
     part = None
+    if dyp.shape[0] > 0 and _pair_ok(E, I, H, need_w, into, dyp.device):
+        # dg and du side by side: their two weight gradients are one grouped product
+        dgu, part = ops.gemm_dgrad_down_packed(dyp, w2b, g, u, offs, gate_blocks)
+        dxp = ops.gemm_dgrad_gateup_packed(dgu, w1b, w3b, offs)
+        dw2 = _wgrad(dyp, act, offs, E, wdtype, need_w[2], into[2])
+        p1, p3 = into[0], into[1]
+        if p1 is None:
+            dw1, dw3 = ops.gemm_wgrad_pair(dgu, xp, offs, E, wdtype)
+        elif p1.grad is None:
+            p1.grad, p3.grad = ops.gemm_wgrad_pair(dgu, xp, offs, E, p1.dtype)
+            dw1 = dw3 = None
+        else:
+            ops.gemm_wgrad_pair(dgu, xp, offs, E, p1.grad.dtype, out1=p1.grad, out3=p3.grad)
+            dw1 = dw3 = None
+        return dxp, dw1, dw3, dw2, part
     if gate_blocks:
         dg, du, part = ops.gemm_dgrad_down(dyp, w2b, g, u, offs, dgate_blocks=True)
     else:

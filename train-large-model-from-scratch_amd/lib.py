@@ -32,6 +32,9 @@ SIGNATURES = {
     "moe_dgates_from_blocks": (_int, [_vp, _i64, _vp, _vp, _i64, _vp, _vp]),
     "moe_gemm_dgrad_gateup": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp]),
     "moe_gemm_wgrad": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _int, _int, _vp]),
+    "moe_gemm_dgrad_down_swiglu_bwd_packed": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _vp]),
+    "moe_gemm_dgrad_gateup_packed": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp]),
+    "moe_gemm_wgrad_pair": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _int, _int, _vp]),
     "moe_segment_offsets": (_int, [_vp, _i64, _i64, _vp, _vp]),
     "moe_combine_fwd": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp, _int, _vp]),
     "moe_combine_bwd": (_int, [_vp, _int, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _vp]),

@@ -168,6 +168,41 @@ def gemm_wgrad(a, b, offs, E: int, dtype: torch.dtype, out: torch.Tensor | None 
     return out
 
 
+def gemm_dgrad_down_packed(dyp, w2, g, u, offs, dgate_blocks: bool = False):
+    """gemm_dgrad_down with dg and du side by side in one buffer: -> dgu bf16 [R, 2I] (row =
+    [dg row | du row]) and, with `dgate_blocks`, the block sums (else None)."""
+    R, H = dyp.shape
+    E, _, I = w2.shape
+    dgu = torch.empty(R, 2 * I, dtype=torch.bfloat16, device=dyp.device)
+    L = _lib.load()
+    part = torch.empty(L.cdll.moe_dgate_blocks(I), R, dtype=torch.float32, device=dyp.device) if dgate_blocks else None
+    L.call("moe_gemm_dgrad_down_swiglu_bwd_packed", _p(dyp), _p(w2), _p(g), _p(u), _p(offs), E, R, H, I,
+           _p(dgu), _p(part), _stream())
+    return dgu, part
+
+
+def gemm_dgrad_gateup_packed(dgu, w1, w3, offs):
+    R = dgu.shape[0]
+    E, I, H = w1.shape
+    dxp = torch.empty(R, H, dtype=torch.bfloat16, device=dgu.device)
+    _lib.load().call("moe_gemm_dgrad_gateup_packed", _p(dgu), _p(w1), _p(w3), _p(offs), E, R, H, I, _p(dxp), _stream())
+    return dxp
+
+
+def gemm_wgrad_pair(dgu, xp, offs, E: int, dtype: torch.dtype, out1=None, out3=None):
+    """dW1[e] (+)= dg[rows e]^T xp[rows e], dW3[e] (+)= du[rows e]^T xp[rows e] from dgu = [dg | du] in
+    one launch; I % 256 == 0.  `out1`/`out3` (both or neither) accumulate."""
+    R, I2 = dgu.shape
+    I, H = I2 // 2, xp.shape[1]
+    acc = out1 is not None
+    if not acc:
+        out1 = torch.empty(E, I, H, dtype=dtype, device=dgu.device)
+        out3 = torch.empty(E, I, H, dtype=dtype, device=dgu.device)
+    _lib.load().call("moe_gemm_wgrad_pair", _p(dgu), _p(xp), _p(offs), E, R, I, H, _p(out1), _p(out3), _dt(out1),
+                     1 if acc else 0, _stream())
+    return out1, out3
+
+
 def segment_offsets(offs: torch.Tensor, E: int, S: int) -> torch.Tensor:
     """offs int32 [E+1] -> int32 [E*S+1]: every expert's rows cut into S equal parts."""
     seg = torch.empty(E * S + 1, dtype=torch.int32, device=offs.device)
