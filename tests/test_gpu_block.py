@@ -143,3 +143,31 @@ def test_config5_real_shape_moe_inside_block(pkg, lib):
     for u, v in zip([out_a.detach()] + grads_a, [out_b.detach()] + grads_b):
         rel = ((u - v).norm() / u.norm().clamp_min(1e-30)).item()
         assert rel < 2e-2, rel
+
+
+@pytest.mark.parametrize("fused", [False, True])
+def test_block_under_deterministic_algorithms(pkg, lib, fused):
+    """The trainer's `--deterministic` switch (utils/training.py:82,
+    `torch.use_deterministic_algorithms(True)`): nothing in the layer's path raises under it
+    (torch then also fills every `torch.empty` with NaN, so a kernel that left part of an output
+    unwritten would show), and two steps give the same bits."""
+    torch.use_deterministic_algorithms(True)
+    try:
+        cfg = pkg.ModelConfig(hidden_size=256, num_attention_heads=4, num_key_value_heads=2, num_experts=8,
+                              num_experts_per_tok=2, moe_intermediate_size=256, init_std=0.05, use_moe=True)
+        blk = pkg.Block(cfg, 2, fused_prenorm=fused)
+        g = torch.Generator().manual_seed(5)
+        x = torch.randn(2, 128, 256, generator=g).cuda().requires_grad_(True)
+        dy = torch.randn(2, 128, 256, generator=g).cuda()
+        runs = []
+        for _ in range(2):
+            blk.zero_grad(set_to_none=True)
+            x.grad = None
+            with torch.autocast("cuda", dtype=torch.bfloat16):
+                out = blk(x)
+            out.backward(dy)
+            runs.append([out.detach().clone(), x.grad.clone()] + [p.grad.clone() for p in blk.parameters()])
+        assert all(torch.isfinite(t).all() for t in runs[0])
+        assert all(torch.equal(a, b) for a, b in zip(*runs))
+    finally:
+        torch.use_deterministic_algorithms(False)
