@@ -385,6 +385,26 @@ def test_bf16_emulation_of_the_rows_entry_matches_the_layer_emulation():
         assert torch.equal(br[n], be[n]), n
 
 
+def test_oracle_reproduces_its_committed_fixture():
+    """tests/golden/oracle_tiny.npz holds what the oracle computed (both modes, forward and
+    backward) on seeded tiny inputs when the fixture was made: an edit that changes what the
+    oracle computes fails here until the fixture is regenerated on purpose."""
+    import importlib.util
+    import os
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    spec = importlib.util.spec_from_file_location("make_oracle_fixture", os.path.join(here, "make_oracle_fixture.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    want = np.load(os.path.join(here, "oracle_tiny.npz"))
+    got = mod.compute()
+    assert set(want.files) == set(got)
+    for k in want.files:
+        if want[k].dtype.kind in "iu":
+            assert np.array_equal(want[k], got[k]), k
+        else:
+            assert np.allclose(want[k], got[k], rtol=1e-5, atol=1e-6), k
+
+
 # ----------------------------------------------------------------------------- block oracle
 def test_block_oracle_pieces():
     from oracle import block_oracle as B
