@@ -103,3 +103,27 @@ def test_registered_operators_propagate_shapes_without_a_gpu():
             d = traced.ffn_bwd(out, xp, g, u, act, gates, ids, offs, p2r, r2p, *wb, k, True, False, wdt == f32)
             assert [tuple(t.shape) for t in d] == [(T, H), (T, E)] + [tuple(w.shape) for w in ws]
             assert [t.dtype for t in d] == [f32, bf, wdt, wdt, wdt]
+
+
+def test_mfu_table_for_amd_parts(monkeypatch):
+    """`profile.py` mirrors utils/profile.py:3-48 for AMD Instinct parts: same function names,
+    arguments and return values, so the reference's MFU line works on an MI355X."""
+    pkg = load_pkg()
+    prof = pkg.profile
+    assert prof.peak_for_device_name("AMD Instinct MI355X", "bf16") == 2.5e15
+    assert prof.peak_for_device_name("AMD Instinct MI355X", "FP8") == 5.0e15
+    assert prof.peak_for_device_name("AMD Instinct MI300X", "bf16") == 1307.4e12
+    assert prof.peak_for_device_name("NVIDIA H100", "bf16") == 0.0
+    assert set(prof.GPU_PEAK_FLOPS["MI355X"]) >= {"fp32", "fp16", "bf16"}   # the reference's keys
+    monkeypatch.setattr(torch.cuda, "get_device_name", lambda i=0: "AMD Instinct MI355X")
+    monkeypatch.setattr(torch.cuda, "device_count", lambda: 8)
+    assert prof.get_gpu_peak_flops("bf16") == 2.5e15
+    assert prof.get_gpu_peak_flops("bf16", per_device=False) == 8 * 2.5e15
+
+    class Model:
+        def get_flops_per_fwd_bwd(self, batch_size, seq_len):
+            return 1.0e15 * batch_size
+
+    mfu, achieved, peak = prof.compute_mfu(Model(), batch_size=2, seq_len=4096, time=2.0, ga=4)
+    assert peak == 2.5e15 and achieved == 4.0e15 and abs(mfu - 1.6) < 1e-12
+    assert prof.compute_mfu(Model(), 1, 1, 0.0)[0] == 0
