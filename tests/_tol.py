@@ -29,8 +29,6 @@ far from the literal bound each tensor was.
 """
 import os
 
-import torch
-
 RTOL = ATOL = 1e-2
 
 # Largest fraction of elements allowed outside the LITERAL bound |d| <= 1e-2 + 1e-2*|ref|,
