@@ -28,12 +28,16 @@ HBM_PEAK_GBS = 8000.0
 # are in profiles/grouped_gemm_cfg3_pmc.txt.  bench.py cannot run the profiler on itself, so
 # the figures are carried here and refreshed whenever that profile is.
 MEASURED_HBM_BYTES_PER_LAUNCH = {
-    (3, "gemm_gateup_swiglu_fwd"): 3.996e9,
-    (3, "gemm_down_fwd"): 1.816e9,
-    (3, "gemm_dgrad_down_swiglu_bwd"): 2.458e9,
-    (3, "gemm_dgrad_gateup"): 3.803e9,
+    (3, "gemm_gateup_swiglu_fwd"): 4.044e9,
+    (3, "gemm_down_fwd"): 1.855e9,
+    (3, "gemm_dgrad_down_swiglu_bwd"): 2.483e9,
+    (3, "gemm_dgrad_gateup"): 3.743e9,
     (3, "gemm_wgrad_down"): 1.074e9,
-    (3, "gemm_wgrad_gate_and_up_pair"): 2.19e9,   # from the average over both weight-gradient launches
+    (3, "gemm_wgrad_gate_and_up_pair"): 2.15e9,   # from the average over both weight-gradient launches
+    # the same kernels under the names of their entry points (as the in-step events see them)
+    (3, "gemm_dgrad_down_swiglu_bwd_packed"): 2.483e9,
+    (3, "gemm_dgrad_gateup_packed"): 3.743e9,
+    (3, "gemm_wgrad_pair"): 2.15e9,
 }
 
 
@@ -51,6 +55,40 @@ def _event_time_ms(torch, fn, iters, warmup):
     e.record()
     torch.cuda.synchronize()
     return s.elapsed_time(e) / iters
+
+
+class _LaunchEvents:
+    """Observer of the library's launches: a pair of HIP events around every entry point,
+    recorded on torch's current stream (the stream the launch is handed), so that each kernel's
+    duration can be read inside the timed steps themselves."""
+
+    def __init__(self, torch):
+        self.torch = torch
+        self.pairs = []
+        self._start = None
+
+    def before(self, name):
+        self._start = self.torch.cuda.Event(enable_timing=True)
+        self._start.record()
+
+    def after(self, name):
+        end = self.torch.cuda.Event(enable_timing=True)
+        end.record()
+        self.pairs.append((name, self._start, end))
+
+    def per_launch_ms(self, steps):
+        """[(entry point, mean ms)] in the order of one step's launches (every step launches the
+        same sequence), after a synchronisation."""
+        n = len(self.pairs) // steps
+        if n == 0 or n * steps != len(self.pairs):
+            return []
+        if any(self.pairs[i][0] != self.pairs[i % n][0] for i in range(len(self.pairs))):
+            return []
+        out = []
+        for j in range(n):
+            ms = [self.pairs[i][1].elapsed_time(self.pairs[i][2]) for i in range(j, len(self.pairs), n)]
+            out.append((self.pairs[j][0], sum(ms) / len(ms)))
+        return out
 
 
 def _moe_dominant_kernel(torch, P, s, x_bf16, wr_bf16, ws_bf16):
@@ -298,6 +336,11 @@ def main():
                          "profiler byte counters)")
     ap.add_argument("--cpu-fraction", type=float, default=1.0,
                     help="fraction of the tokens the CPU baseline sample processes")
+    ap.add_argument("--no-kernel-events", dest="kernel_events", action="store_false",
+                    help="record no HIP events around the launches inside the timed steps")
+    ap.add_argument("--no-kernel-loops", action="store_true",
+                    help="skip the separate back-to-back timing loops of the single kernels and the library's "
+                         "dense reference (a profiler then sees the launches of the steps only)")
     ap.add_argument("--no-others", action="store_true",
                     help="skip the short runs of the other benchmark configurations (field other_configs)")
     args = ap.parse_args()
@@ -361,6 +404,21 @@ def main():
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) * 1e3 / args.steps
     tflops = flops / ms / 1e9
+    # The same K steps once more, now with a pair of HIP events around every launch: each
+    # kernel's duration inside the step.  A region of its own because the 2 x 15 event records
+    # per step cost about 1 % of the step (5.33 against 5.28 ms), which the headline figure
+    # should not carry; only where the step is bound by the GPU (the two large configurations).
+    in_step, ms_events = [], None
+    if args.kernel_events and args.config in (3, 4):
+        watch = _LaunchEvents(torch)
+        P.lib.load().observer = watch
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        ms_events = (time.perf_counter() - t0) * 1e3 / args.steps
+        P.lib.load().observer = None
+        in_step = watch.per_launch_ms(args.steps)
     tokens_per_s = s.T / (ms * 1e-3)
 
     # the same step captured once in a HIP graph and replayed: what a caller gets who removes
@@ -395,96 +453,134 @@ def main():
         del src, dst
 
     # ---------------- per-kernel durations (HIP events), for the roofline object
-    with torch.no_grad():
-        xd = x.detach()
-        w1, w3, w2 = (w.detach() for w in ws)
-        if s.rows_entry:
-            _, offs, p2r, r2p = ops.histogram_scan(ids.to(torch.int32), s.E)
-            kk, gates = 1, None
-        else:
-            logits = F.linear(xd, wr.detach())
-            rids, gates = ops.router_topk(logits, s.k, bias)
-            _, offs, p2r, r2p = ops.histogram_scan(rids, s.E)
-            kk = s.k
-        xp = ops.permute_fwd(xd, p2r, kk, r2p)
-        g, u, act = ops.gemm_gateup(xp, w1, w3, offs, True)
-        y = ops.gemm_down(act, w2, offs)
-        dyy = dy if dy is not None else torch.randn_like(xd)
-        dyp, _ = ops.combine_bwd(dyy, None, gates, p2r, kk, r2p)
-        routed = gates is not None  # the gate gradients' block sums ride in the dgrad-down kernel
-        # (dg and du side by side in one buffer, as the backward pass keeps them when I % 256 == 0:
-        # their two weight gradients are then one launch)
-        packed = s.I % 256 == 0
-        if packed:
-            dgu = ops.gemm_dgrad_down_packed(dyp, w2, g, u, offs, dgate_blocks=routed)[0]
-            dxp = ops.gemm_dgrad_gateup_packed(dgu, w1, w3, offs)
-            dg = dgu[:, :s.I].contiguous()
-        else:
-            dg, du = ops.gemm_dgrad_down(dyp, w2, g, u, offs, dgate_blocks=routed)[:2]
-            dxp = ops.gemm_dgrad_gateup(dg, du, w1, w3, offs)
-        bf = torch.bfloat16
-        a = 2  # bytes per bf16 element
-        T, R, H, I, E = xd.shape[0], s.R, s.H, s.I, s.E
-        kernels = [
-            # name, callable, algorithmic flops, algorithmic bytes, launches per step
-            ("gemm_gateup_swiglu_fwd", lambda: ops.gemm_gateup(xp, w1, w3, offs, True), 4 * RHI, 0, 1),
-            ("gemm_down_fwd", lambda: ops.gemm_down(act, w2, offs), 2 * RHI, 0, 1),
-            ("gemm_dgrad_down_swiglu_bwd",
-             (lambda: ops.gemm_dgrad_down_packed(dyp, w2, g, u, offs, dgate_blocks=routed)) if packed else
-             (lambda: ops.gemm_dgrad_down(dyp, w2, g, u, offs, dgate_blocks=routed)), 2 * RHI, 0, 1),
-            ("gemm_dgrad_gateup",
-             (lambda: ops.gemm_dgrad_gateup_packed(dgu, w1, w3, offs)) if packed else
-             (lambda: ops.gemm_dgrad_gateup(dg, du, w1, w3, offs)), 4 * RHI, 0, 1),
-            ("gemm_wgrad_down", lambda: ops.gemm_wgrad(dyp, act, offs, E, bf), 2 * RHI, 0, 1),
-            (("gemm_wgrad_gate_and_up_pair", lambda: ops.gemm_wgrad_pair(dgu, xp, offs, E, bf), 4 * RHI, 0, 1) if packed
-             else ("gemm_wgrad_gate_or_up", lambda: ops.gemm_wgrad(dg, xp, offs, E, bf), 2 * RHI, 0, 2)),
-            ("permute_fwd", lambda: ops.permute_fwd(xd, p2r, kk, r2p), 0, T * H * a + R * H * a + R * 4, 1),
-            ("combine_fwd", lambda: ops.combine_fwd(y, gates, r2p, T, kk, xd.dtype), 0,
-             R * H * a + R * 8 + T * H * a, 1),
-            ("combine_bwd", lambda: ops.combine_bwd(dyy, None, gates, p2r, kk, r2p), 0,
-             T * H * a + R * H * a + R * 8, 1),
-            ("permute_bwd", lambda: ops.permute_bwd(dxp, r2p, T, kk, xd.dtype), 0, R * H * a + T * H * a, 1),
-        ]
-        # fp32 master -> bf16 operand cast of one weight stack: not part of this step (the
-        # configuration hands over bf16 weights); the module pays it once per optimizer step
-        # and stack, the reference once per forward and stack
-        w_master = torch.empty(w1.shape, dtype=torch.float32, device=dev).normal_()
-        kernels.append(("cast_f32_bf16_one_weight_stack", lambda: ops.cast_bf16(w_master), 0,
-                        w_master.numel() * 6, 0))
-        per_kernel = []
-        for name, fn, fl, by, launches in kernels:
-            kms = _event_time_ms(torch, fn, 10, 2)
-            rec = {"kernel": name, "ms": round(kms, 4), "launches_per_step": launches}
-            if fl:
-                rec.update(bound="mfma", achieved=round(fl / kms / 1e9, 1), unit="TFLOP/s",
-                           frac=round(fl / kms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4))
+    per_kernel, lib_ref = [], {}
+    if not args.no_kernel_loops:
+        with torch.no_grad():
+            xd = x.detach()
+            w1, w3, w2 = (w.detach() for w in ws)
+            if s.rows_entry:
+                _, offs, p2r, r2p = ops.histogram_scan(ids.to(torch.int32), s.E)
+                kk, gates = 1, None
             else:
-                rec.update(bound="hbm", achieved=round(by / kms / 1e6, 1), unit="GB/s",
-                           frac=round(by / kms / 1e6 / HBM_PEAK_GBS, 4))
-            per_kernel.append(rec)
-        # what the vendor's dense GEMM library reaches on this part on problems of the same size
-        # with none of the layer's structure (one weight for all rows, no ragged groups, no fused
-        # epilogue, one output): the practical ceiling the grouped kernels are measured against
-        lib_ref = {}
-        if True:
-            wd = torch.randn(2 * I, H, device=dev).to(bf) * 0.02
-            wdn = torch.randn(H, I, device=dev).to(bf) * 0.02
-            t_gu = _event_time_ms(torch, lambda: torch.mm(xp, wd.t()), 10, 3)
-            t_dn = _event_time_ms(torch, lambda: torch.mm(act, wdn.t()), 10, 3)
-            lib_ref = {"what": "torch.mm (hipBLASLt) on dense problems of the gate/up and down sizes: "
-                               "[R,H]x[H,2I] and [R,I]x[I,H], bf16, same random data scale",
-                       "gateup_size_tflops": round(4 * RHI / t_gu / 1e9, 1), "down_size_tflops": round(2 * RHI / t_dn / 1e9, 1),
-                       "gateup_size_frac_of_peak": round(4 * RHI / t_gu / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4)}
-            del wd, wdn
+                logits = F.linear(xd, wr.detach())
+                rids, gates = ops.router_topk(logits, s.k, bias)
+                _, offs, p2r, r2p = ops.histogram_scan(rids, s.E)
+                kk = s.k
+            xp = ops.permute_fwd(xd, p2r, kk, r2p)
+            g, u, act = ops.gemm_gateup(xp, w1, w3, offs, True)
+            y = ops.gemm_down(act, w2, offs)
+            dyy = dy if dy is not None else torch.randn_like(xd)
+            dyp, _ = ops.combine_bwd(dyy, None, gates, p2r, kk, r2p)
+            routed = gates is not None  # the gate gradients' block sums ride in the dgrad-down kernel
+            # (dg and du side by side in one buffer, as the backward pass keeps them when I % 256 == 0:
+            # their two weight gradients are then one launch)
+            packed = s.I % 256 == 0
+            if packed:
+                dgu = ops.gemm_dgrad_down_packed(dyp, w2, g, u, offs, dgate_blocks=routed)[0]
+                dxp = ops.gemm_dgrad_gateup_packed(dgu, w1, w3, offs)
+                dg = dgu[:, :s.I].contiguous()
+            else:
+                dg, du = ops.gemm_dgrad_down(dyp, w2, g, u, offs, dgate_blocks=routed)[:2]
+                dxp = ops.gemm_dgrad_gateup(dg, du, w1, w3, offs)
+            bf = torch.bfloat16
+            a = 2  # bytes per bf16 element
+            T, R, H, I, E = xd.shape[0], s.R, s.H, s.I, s.E
+            kernels = [
+                # name, callable, algorithmic flops, algorithmic bytes, launches per step
+                ("gemm_gateup_swiglu_fwd", lambda: ops.gemm_gateup(xp, w1, w3, offs, True), 4 * RHI, 0, 1),
+                ("gemm_down_fwd", lambda: ops.gemm_down(act, w2, offs), 2 * RHI, 0, 1),
+                ("gemm_dgrad_down_swiglu_bwd",
+                 (lambda: ops.gemm_dgrad_down_packed(dyp, w2, g, u, offs, dgate_blocks=routed)) if packed else
+                 (lambda: ops.gemm_dgrad_down(dyp, w2, g, u, offs, dgate_blocks=routed)), 2 * RHI, 0, 1),
+                ("gemm_dgrad_gateup",
+                 (lambda: ops.gemm_dgrad_gateup_packed(dgu, w1, w3, offs)) if packed else
+                 (lambda: ops.gemm_dgrad_gateup(dg, du, w1, w3, offs)), 4 * RHI, 0, 1),
+                ("gemm_wgrad_down", lambda: ops.gemm_wgrad(dyp, act, offs, E, bf), 2 * RHI, 0, 1),
+                (("gemm_wgrad_gate_and_up_pair", lambda: ops.gemm_wgrad_pair(dgu, xp, offs, E, bf), 4 * RHI, 0, 1) if packed
+                 else ("gemm_wgrad_gate_or_up", lambda: ops.gemm_wgrad(dg, xp, offs, E, bf), 2 * RHI, 0, 2)),
+                ("permute_fwd", lambda: ops.permute_fwd(xd, p2r, kk, r2p), 0, T * H * a + R * H * a + R * 4, 1),
+                ("combine_fwd", lambda: ops.combine_fwd(y, gates, r2p, T, kk, xd.dtype), 0,
+                 R * H * a + R * 8 + T * H * a, 1),
+                ("combine_bwd", lambda: ops.combine_bwd(dyy, None, gates, p2r, kk, r2p), 0,
+                 T * H * a + R * H * a + R * 8, 1),
+                ("permute_bwd", lambda: ops.permute_bwd(dxp, r2p, T, kk, xd.dtype), 0, R * H * a + T * H * a, 1),
+            ]
+            # fp32 master -> bf16 operand cast of one weight stack: not part of this step (the
+            # configuration hands over bf16 weights); the module pays it once per optimizer step
+            # and stack, the reference once per forward and stack
+            w_master = torch.empty(w1.shape, dtype=torch.float32, device=dev).normal_()
+            kernels.append(("cast_f32_bf16_one_weight_stack", lambda: ops.cast_bf16(w_master), 0,
+                            w_master.numel() * 6, 0))
+            per_kernel = []
+            for name, fn, fl, by, launches in kernels:
+                kms = _event_time_ms(torch, fn, 10, 2)
+                rec = {"kernel": name, "ms": round(kms, 4), "launches_per_step": launches}
+                if fl:
+                    rec.update(bound="mfma", achieved=round(fl / kms / 1e9, 1), unit="TFLOP/s",
+                               frac=round(fl / kms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4))
+                else:
+                    rec.update(bound="hbm", achieved=round(by / kms / 1e6, 1), unit="GB/s",
+                               frac=round(by / kms / 1e6 / HBM_PEAK_GBS, 4))
+                per_kernel.append(rec)
+            # what the vendor's dense GEMM library reaches on this part on problems of the same size
+            # with none of the layer's structure (one weight for all rows, no ragged groups, no fused
+            # epilogue, one output): the practical ceiling the grouped kernels are measured against
+            lib_ref = {}
+            if True:
+                wd = torch.randn(2 * I, H, device=dev).to(bf) * 0.02
+                wdn = torch.randn(H, I, device=dev).to(bf) * 0.02
+                t_gu = _event_time_ms(torch, lambda: torch.mm(xp, wd.t()), 10, 3)
+                t_dn = _event_time_ms(torch, lambda: torch.mm(act, wdn.t()), 10, 3)
+                lib_ref = {"what": "torch.mm (hipBLASLt) on dense problems of the gate/up and down sizes: "
+                                   "[R,H]x[H,2I] and [R,I]x[I,H], bf16, same random data scale",
+                           "gateup_size_tflops": round(4 * RHI / t_gu / 1e9, 1), "down_size_tflops": round(2 * RHI / t_dn / 1e9, 1),
+                           "gateup_size_frac_of_peak": round(4 * RHI / t_gu / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4)}
+                del wd, wdn
     gemms = [r for r in per_kernel if r["bound"] == "mfma"]
     if not s.backward:
         gemms = gemms[:2]
-    dominant = max(gemms, key=lambda r: r["ms"] * r["launches_per_step"])
-    gemm_ms = sum(r["ms"] * r["launches_per_step"] for r in gemms)
-    roofline = {"kernel": dominant["kernel"], "bound": "mfma", "achieved": dominant["achieved"],
-                "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": dominant["frac"], "traffic": None,
-                "all_gemms_tflops": round(flops / gemm_ms / 1e9, 1),
-                "all_gemms_frac": round(flops / gemm_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4)}
+    roofline = {"kernel": None, "bound": "mfma", "achieved": None, "peak": MFMA_BF16_PEAK_TFLOPS,
+                "unit": "TFLOP/s", "frac": None, "traffic": None}
+    dominant = None
+    if gemms:
+        dominant = max(gemms, key=lambda r: r["ms"] * r["launches_per_step"])
+        gemm_ms = sum(r["ms"] * r["launches_per_step"] for r in gemms)
+        roofline.update(kernel=dominant["kernel"], achieved=dominant["achieved"], frac=dominant["frac"],
+                        all_gemms_tflops=round(flops / gemm_ms / 1e9, 1),
+                        all_gemms_frac=round(flops / gemm_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4))
+
+    # the same kernels inside the timed steps (events around every launch): these are the
+    # durations the roofline object reports where they exist; the figures from the separate
+    # loops above stay beside them
+    in_step_recs = []
+    if in_step:
+        gemm_flops_of = {"moe_gemm_gateup_swiglu_fwd": 4, "moe_gemm_down_fwd": 2, "moe_gemm_dgrad_down_swiglu_bwd": 2,
+                         "moe_gemm_dgrad_down_swiglu_bwd_dgate": 2, "moe_gemm_dgrad_down_swiglu_bwd_packed": 2,
+                         "moe_gemm_dgrad_gateup": 4, "moe_gemm_dgrad_gateup_packed": 4, "moe_gemm_wgrad_pair": 4,
+                         "moe_gemm_wgrad": 2}
+        # moe_gemm_wgrad also serves the router's small split-k product: only launches of at least a
+        # tenth of the longest one are the experts' weight gradients
+        longest_wgrad = max([m for n, m in in_step if n == "moe_gemm_wgrad"], default=0.0)
+        for name, kms in in_step:
+            rec = {"entry": name, "ms": round(kms, 4)}
+            f = gemm_flops_of.get(name)
+            if f and not (name == "moe_gemm_wgrad" and kms < 0.1 * longest_wgrad):
+                rec.update(achieved=round(f * RHI / kms / 1e9, 1), unit="TFLOP/s",
+                           frac=round(f * RHI / kms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4))
+            in_step_recs.append(rec)
+        g_in = [r for r in in_step_recs if "frac" in r]
+        if g_in:
+            dom = max(g_in, key=lambda r: r["ms"])
+            g_ms = sum(r["ms"] for r in g_in)
+            roofline.update(
+                kernel=dom["entry"].replace("moe_", "", 1), achieved=dom["achieved"], frac=dom["frac"],
+                ms=dom["ms"],
+                measured=f"HIP events around this launch in each of {args.steps} steps that follow the timed "
+                         f"ones ({round(ms_events, 4)} ms per step with the events)",
+                achieved_back_to_back=dominant["achieved"] if dominant else None,
+                all_gemms_tflops=round(flops / g_ms / 1e9, 1),
+                all_gemms_frac=round(flops / g_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
+                launches_ms_sum=round(sum(r["ms"] for r in in_step_recs), 4))
 
     roofline["traffic"] = MEASURED_HBM_BYTES_PER_LAUNCH.get((args.config, roofline["kernel"]))
     roofline["traffic_source"] = ("rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this benchmark, "
@@ -521,7 +617,8 @@ def main():
         "tokens_per_s": round(tokens_per_s, 1),
         "ms_per_step_graph_replay": None if ms_graph is None else round(ms_graph, 4),
         "mfma_peak_frac_whole_step": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
-        "roofline": roofline, "cpu_baseline": cpu, "kernels": per_kernel, "library_dense_reference": lib_ref,
+        "roofline": roofline, "cpu_baseline": cpu, "kernels": per_kernel, "kernels_in_step": in_step_recs or None,
+        "library_dense_reference": lib_ref,
         "other_configs": others,
     }
     print(json.dumps(line), flush=True)

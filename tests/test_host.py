@@ -127,3 +127,30 @@ def test_mfu_table_for_amd_parts(monkeypatch):
     mfu, achieved, peak = prof.compute_mfu(Model(), batch_size=2, seq_len=4096, time=2.0, ga=4)
     assert peak == 2.5e15 and achieved == 4.0e15 and abs(mfu - 1.6) < 1e-12
     assert prof.compute_mfu(Model(), 1, 1, 0.0)[0] == 0
+
+
+def test_launch_observer_sees_every_entry_point_call():
+    """`MoELib.observer` is called around every entry point (bench.py hangs HIP events on it).
+    A null pointer is refused by the argument checks before anything touches a GPU, so this
+    runs on the CPU."""
+    pkg = load_pkg()
+    L = pkg.lib.load()
+    seen = []
+
+    class Obs:
+        def before(self, name):
+            seen.append(("before", name))
+
+        def after(self, name):
+            seen.append(("after", name))
+
+    L.observer = Obs()
+    try:
+        with pytest.raises(pkg.lib.MoELibError, match="MOE_ERR_NULL"):
+            L.call("moe_cast_f32_bf16", None, None, 8, None)
+        L.call("moe_cast_f32_bf16", None, None, 0, None)  # nothing to do: returns 0
+    finally:
+        L.observer = None
+    assert seen == [("before", "moe_cast_f32_bf16"), ("after", "moe_cast_f32_bf16")] * 2
+    L.call("moe_cast_f32_bf16", None, None, 0, None)
+    assert len(seen) == 4

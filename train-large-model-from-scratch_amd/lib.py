@@ -68,9 +68,17 @@ class MoELib:
             fn = getattr(self.cdll, name)  # AttributeError if the symbol is missing
             fn.restype, fn.argtypes = res, args
         self.abi_version = self.cdll.moe_abi_version()
+        # Optional observer of the launches (a profiling aid): an object with before(name) and
+        # after(name), called around every entry point, e.g. to record events on the stream.
+        self.observer = None
 
     def call(self, name: str, *args):
+        obs = self.observer
+        if obs is not None:
+            obs.before(name)
         rc = getattr(self.cdll, name)(*args)
+        if obs is not None:
+            obs.after(name)
         if rc != 0:
             what = ERRORS.get(rc, f"hipError_t {rc}" if rc > 0 else f"code {rc}")
             raise MoELibError(f"{name} failed: {what}")
