@@ -52,16 +52,19 @@ def topk_select(logits: torch.Tensor, k: int) -> tuple[np.ndarray, torch.Tensor]
     """Canonical top-k of mlp.py:101: ids[T,k] int64 and the selected logits [T,k].
 
     Slots are in descending-logit order (torch.topk's `sorted=True` default); equal
-    logits are ordered by ascending expert index.
+    logits are ordered by ascending expert index; a NaN ranks above every number, as it
+    does for torch.topk.
     pinned by: brute-force insertion on tiny inputs, equality with torch.topk on rows
-    without ties, selected-value multiset equality on rows with ties.
+    without ties (rows with one NaN, with +-inf included), selected-value multiset equality
+    on rows with ties.
     """
     lg = logits.detach().to(torch.float64).cpu().numpy()  # exact for bf16/fp32 values
     T, E = lg.shape
     assert 0 < k <= E
     eidx = np.broadcast_to(np.arange(E), (T, E))
-    # lexsort: last key is primary.  primary = -logit (descending), secondary = index.
-    order = np.lexsort((eidx, -lg), axis=-1)[:, :k].astype(np.int64)
+    nan = np.isnan(lg)
+    # lexsort: last key is primary.  NaNs first, then -logit (descending), then the index.
+    order = np.lexsort((eidx, np.where(nan, 0.0, -lg), ~nan), axis=-1)[:, :k].astype(np.int64)
     sel = torch.gather(logits, 1, torch.from_numpy(order).to(logits.device))
     return order, sel
 

@@ -58,6 +58,45 @@ def test_router_topk_bit_exact(ops, T, E, k, dtype, quant):
     assert torch.allclose(gates.cpu().reshape(T, k), og, atol=1e-6, rtol=1e-5)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_router_topk_non_finite_logits(ops, dtype):
+    """Experts masked with -inf (fewer finite logits than k included), a +inf logit, a row of
+    -inf and a NaN: selection and gates as torch.topk + softmax give them (mlp.py:101-102) --
+    masked experts are taken last, lowest index first, with gate 0; a row whose softmax is
+    NaN in the reference is NaN here; ids stay distinct and in range; other rows are untouched."""
+    T, E, k = 256, 64, 8
+    g = torch.Generator().manual_seed(77)
+    logits = torch.randn(T, E, generator=g)
+    inf = float("inf")
+    logits[0, 5:] = -inf                       # 5 finite logits, k = 8
+    logits[1, ::2] = -inf                      # half of the experts masked
+    logits[2, 17] = inf
+    logits[3, :] = -inf
+    logits[4, 9] = float("nan")
+    logits[5, :] = 0.0
+    logits[5, 60:] = -inf
+    clean = logits.clone()
+    logits = logits.to(dtype)
+    ids, gates = ops.router_topk(logits.cuda(), k)
+    ids = ids.cpu().numpy().reshape(T, k)
+    gates = gates.cpu().reshape(T, k)
+    assert ids.min() >= 0 and ids.max() < E
+    assert all(len(set(row)) == k for row in ids)
+    oid, osel = O.topk_select(logits, k)
+    assert np.array_equal(ids, oid.astype(np.int32))
+    og = O.gates_from_selected(osel)
+    assert torch.allclose(gates, og, atol=1e-6, rtol=1e-5, equal_nan=True)
+    assert torch.isnan(gates[2]).all() and torch.isnan(gates[3]).all() and torch.isnan(gates[4]).all()
+    assert ids[4, 0] == 9                      # a NaN ranks above every number, as for torch.topk,
+    #                                            whatever its sign (torch's CPU cast to bf16 sets it)
+    assert torch.equal(gates[0, 5:], torch.zeros(3)) and sorted(ids[0, :5]) == [0, 1, 2, 3, 4]
+    assert list(ids[0, 5:]) == [5, 6, 7]
+    assert torch.isfinite(gates[6:]).all()
+    # the library routine on the rows where it is unambiguous (no ties among the selected)
+    if dtype == torch.float32:                 # (bf16 rows hold ties, which the library orders its own way)
+        assert np.array_equal(ids[6:], torch.topk(clean[6:], k).indices.numpy())
+
+
 def test_router_topk_with_bias(ops):
     T, E, k = 4096, 8, 2
     g = torch.Generator().manual_seed(5)

@@ -70,6 +70,28 @@ def test_topk_matches_torch_on_tie_free_rows():
     assert all(len(set(r)) == k for r in ids.tolist())
 
 
+def test_topk_non_finite_matches_torch():
+    """NaN ranks above every number and -inf below (torch.topk's order, mlp.py:101), whatever the
+    NaN's sign bit; checked against the library routine on fp32 rows without ties."""
+    g = torch.Generator().manual_seed(31)
+    logits = torch.randn(64, 32, generator=g)
+    inf = float("inf")
+    logits[0, 3] = float("nan")
+    logits[1, 7] = torch.tensor([0xffc00000 - (1 << 32)], dtype=torch.int32).view(torch.float32).item()  # sign set
+    logits[2, 5] = inf
+    logits[3, 10:] = -inf            # 10 finite logits, k = 8: still no tie among the selected
+    logits[4, 0] = float("nan")
+    logits[4, 1] = inf
+    k = 8
+    ids, sel = O.topk_select(logits, k)
+    tv, ti = torch.topk(logits, k, dim=-1)
+    assert np.array_equal(ids, ti.numpy())
+    assert torch.equal(torch.nan_to_num(sel, nan=123.0), torch.nan_to_num(tv, nan=123.0))
+    assert ids[0, 0] == 3 and ids[1, 0] == 7 and ids[4, :2].tolist() == [0, 1]
+    gates = O.gates_from_selected(sel)
+    assert torch.isnan(gates[[0, 1, 2, 4]]).all() and torch.isfinite(gates[3]).all()
+
+
 def test_gates_invariants():
     g = torch.Generator().manual_seed(4)
     logits = torch.randn(64, 16, generator=g)

@@ -7,7 +7,9 @@
 __device__ __forceinline__ uint32_t moe_orderable(float v) {
   v += 0.0f;  // -0.0 -> +0.0 so that the two compare equal, as they do for torch.topk
   uint32_t u = __builtin_bit_cast(uint32_t, v);
-  return u ^ ((u >> 31) ? 0xffffffffu : 0x80000000u);
+  // a NaN of either sign ranks above every number, as it does for torch.topk (and maps back
+  // to a NaN, so the token's gates are NaN as the reference's are)
+  return (v != v) ? 0xffffffffu : u ^ ((u >> 31) ? 0xffffffffu : 0x80000000u);
 }
 __device__ __forceinline__ float moe_from_orderable(uint32_t u) {
   u ^= ((u >> 31) ? 0x80000000u : 0xffffffffu);
