@@ -599,3 +599,42 @@ def test_routed_moe_is_router_linear_plus_moe_ffn(P, x_dtype):
     torch.autograd.backward([o3, lg3], [dy, dl])
     extra = dl.float().cpu() @ inp["wr"].float()
     check("dx with a logits gradient", x3.grad, b["dx"] + extra, (be["dx"] + extra).to(x_dtype).float(), say=_say)
+
+
+@pytest.mark.parametrize("entry", ENTRIES + ("experts_rows", "module", "module_prenorm"))
+def test_no_tokens(P, entry):
+    """An empty batch (the reference handles it: every count is zero, `max_tokens` is 0 and the
+    padded products have no rows, mlp.py:126-158): empty output of the right shape and dtype,
+    exact-zero weight gradients, an empty input gradient; nothing faults."""
+    H, I, E, k = 64, 32, 4, 2
+    dev = "cuda"
+    g = torch.Generator().manual_seed(3)
+    r = lambda *s_: (torch.randn(*s_, generator=g) * 0.1).to(torch.bfloat16).to(dev).requires_grad_(True)
+    x, wr, w1, w3, w2 = r(0, H), r(E, H), r(E, I, H), r(E, I, H), r(E, H, I)
+    if entry == "moe_ffn":
+        out = P.moe_ffn(x, F.linear(x, wr), w1, w3, w2, k)
+    elif entry == "routed_moe":
+        out, logits = P.routed_moe(x, wr, w1, w3, w2, k)
+        assert logits.shape == (0, E)
+    elif entry == "experts_rows":
+        out = P.experts_rows(x, torch.empty(0, dtype=torch.int32, device=dev), w1, w3, w2)
+    else:
+        cfg = P.ModelConfig(hidden_size=H, intermediate_size=I, num_experts=E, num_experts_per_tok=k)
+        m = P.MoE(cfg).to(dev)
+        xb = torch.zeros(2, 0, H, device=dev, requires_grad=True)
+        norm = P.block.RMSNorm(H).to(dev)
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            out, logits = m(xb) if entry == "module" else m.forward_prenorm(xb, norm)
+        assert out.shape == (2, 0, H) and out.dtype == torch.float32 and logits.shape == (2, 0, E)
+        out.sum().backward()
+        for p_ in (m.experts_gate_weights, m.experts_up_weights, m.experts_down_weights):
+            assert p_.grad is not None and not p_.grad.any()
+        if entry == "module_prenorm":
+            assert norm.weight.grad is not None and not norm.weight.grad.any()
+        return
+    assert out.shape == (0, H) and out.dtype == torch.bfloat16
+    out.backward(torch.empty_like(out))
+    assert x.grad is not None and x.grad.shape == (0, H)
+    for w in (w1, w3, w2):
+        assert w.grad is not None and not w.grad.any()
+    torch.cuda.synchronize()

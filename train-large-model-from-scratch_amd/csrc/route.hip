@@ -91,11 +91,11 @@ int dispatch_vpl(int64_t E, F&& f) {
 extern "C" int moe_router_topk_fwd(const void* logits, int logits_dtype, const float* bias,
                                    int64_t T, int64_t E, int64_t k, int32_t* ids_out,
                                    float* gates_out, void* stream) {
-  if (!logits || !ids_out || !gates_out) return MOE_ERR_NULL;
   if (T < 0 || E <= 0 || k <= 0 || k > E) return MOE_ERR_SHAPE;
   if (E > MOE_MAX_EXPERTS || k > MOE_MAX_TOPK || T > (int64_t)1 << 30) return MOE_ERR_LIMIT;
   if (logits_dtype != MOE_DT_BF16 && logits_dtype != MOE_DT_F32) return MOE_ERR_DTYPE;
-  if (T == 0) return 0;
+  if (T == 0) return 0;  // nothing to read or write: empty buffers may be null
+  if (!logits || !ids_out || !gates_out) return MOE_ERR_NULL;
   const dim3 block(256), grid((unsigned)((T + 3) / 4));
   hipStream_t s = (hipStream_t)stream;
   return dispatch_vpl(E, [&](auto vpl) {
@@ -113,11 +113,11 @@ extern "C" int moe_router_topk_fwd(const void* logits, int logits_dtype, const f
 extern "C" int moe_router_topk_bwd(const float* gates, const float* dgates, const int32_t* ids,
                                    int64_t T, int64_t E, int64_t k, void* dlogits,
                                    int dlogits_dtype, void* stream) {
-  if (!gates || !dgates || !ids || !dlogits) return MOE_ERR_NULL;
   if (T < 0 || E <= 0 || k <= 0 || k > E) return MOE_ERR_SHAPE;
   if (E > MOE_MAX_EXPERTS || k > MOE_MAX_TOPK || T > (int64_t)1 << 30) return MOE_ERR_LIMIT;
   if (dlogits_dtype != MOE_DT_BF16 && dlogits_dtype != MOE_DT_F32) return MOE_ERR_DTYPE;
   if (T == 0) return 0;
+  if (!gates || !dgates || !ids || !dlogits) return MOE_ERR_NULL;
   const dim3 block(256), grid((unsigned)((T + 3) / 4));
   hipStream_t s = (hipStream_t)stream;
   return dispatch_vpl(E, [&](auto vpl) {
