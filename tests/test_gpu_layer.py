@@ -638,3 +638,49 @@ def test_no_tokens(P, entry):
     for w in (w1, w3, w2):
         assert w.grad is not None and not w.grad.any()
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("entry", ENTRIES + ("experts_rows",))
+def test_strided_and_unaligned_inputs(P, entry):
+    """Inputs that are views -- every other row of a larger tensor, a view that starts 6 bytes
+    into an aligned block, a gradient that is such a view -- give the same bits as their dense
+    copies (the reference takes any strides: its first step is a reshape, mlp.py:98-99)."""
+    T, H, I, E, k = 96, 128, 64, 4, 2
+    dev = "cuda"
+    g = torch.Generator().manual_seed(9)
+    rnd = lambda *s_, std=1.0: (torch.randn(*s_, generator=g) * std).to(torch.bfloat16).to(dev)
+    x_d, dy_d = rnd(T, H), rnd(T, H)
+    wr, w1, w3, w2 = rnd(E, H, std=0.3), rnd(E, I, H, std=0.1), rnd(E, I, H, std=0.1), rnd(E, H, I, std=0.1)
+    ids = torch.randint(0, E, (T,), generator=g).to(dev)
+
+    def views():
+        big = torch.zeros(2 * T, H, dtype=torch.bfloat16, device=dev)
+        big[::2] = x_d
+        flat = torch.zeros(T * H + 8, dtype=torch.bfloat16, device=dev)
+        flat[3:3 + T * H] = dy_d.reshape(-1)
+        xv, dyv = big[::2], flat[3:3 + T * H].view(T, H)
+        assert not xv.is_contiguous() and dyv.data_ptr() % 16 != 0
+        return xv, dyv
+
+    def run(x, dy):
+        x = x.detach().requires_grad_(True)
+        ws = [w.detach().clone().requires_grad_(True) for w in (w1, w3, w2)]
+        if entry == "moe_ffn":
+            out = P.moe_ffn(x, F.linear(x, wr), *ws, k)
+        elif entry == "routed_moe":
+            out, _ = P.routed_moe(x, wr, *ws, k)
+        else:
+            out = P.experts_rows(x, ids, *ws)
+        out.backward(dy)
+        return [out.detach(), x.grad] + [w.grad for w in ws]
+
+    xv, dyv = views()
+    a, b = run(x_d, dy_d), run(xv, dyv)
+    for t_a, t_b in zip(a, b):
+        assert torch.equal(t_a, t_b)
+    # x itself may also start off the 16-byte grid
+    flat = torch.zeros(T * H + 8, dtype=torch.bfloat16, device=dev)
+    flat[5:5 + T * H] = x_d.reshape(-1)
+    c = run(flat[5:5 + T * H].view(T, H), dy_d)
+    for t_a, t_c in zip(a, c):
+        assert torch.equal(t_a, t_c)

@@ -62,6 +62,13 @@ class _RouterLinear(torch.autograd.Function):
         return dx, dw
 
 
+def _dense(t: torch.Tensor) -> torch.Tensor:
+    """Contiguous and 16-byte aligned, as the kernels need their buffers: a copy only for a
+    strided view or a view that starts in the middle of an aligned block."""
+    t = t.contiguous()
+    return t if t.data_ptr() % 16 == 0 else t.clone()
+
+
 def _router_wgrad(dlogits, x, w_dtype):
     """dWr = dlogits^T x for dlogits [T,E], x [T,H]."""
     T, H = x.shape
@@ -81,7 +88,7 @@ def _router_wgrad(dlogits, x, w_dtype):
         if len(_split_offsets) > 64:
             _split_offsets.clear()
         _split_offsets[key] = offs
-    part = ops.gemm_wgrad(dlogits.contiguous(), x.contiguous(), offs, S, torch.float32)
+    part = ops.gemm_wgrad(_dense(dlogits), _dense(x), offs, S, torch.float32)
     return part.sum(0).to(w_dtype)
 
 
@@ -214,10 +221,10 @@ class _MoEFFN(torch.autograd.Function):
     def forward(ctx, x, logits, w1, w3, w2, k, bias, shadows, grad_params):
         T, H = x.shape
         E = logits.shape[1]
-        x = x.contiguous()
-        logits = logits.contiguous()
+        x = _dense(x)
+        logits = _dense(logits)
         shadows = shadows or (None, None, None)
-        w1b, w3b, w2b = (sh if sh is not None else ops.cast_bf16(w.contiguous())
+        w1b, w3b, w2b = (sh if sh is not None else ops.cast_bf16(_dense(w))
                          for w, sh in zip((w1, w3, w2), shadows))
         ids, gates = ops.router_topk(logits, k, bias)
         counts, offs, pos_to_row, row_to_pos = ops.histogram_scan(ids, E)
@@ -244,7 +251,7 @@ class _MoEFFN(torch.autograd.Function):
         if dout is None:
             dout = torch.zeros(ctx.out_shape, dtype=ctx.x_dtype, device=xp.device)
         T = dout.shape[0]
-        dout = dout.contiguous()
+        dout = _dense(dout)
         if dout.dtype not in (torch.bfloat16, torch.float32):
             dout = dout.float()
         dyp, _ = ops.combine_bwd(dout, None, gates, pos_to_row, k, row_to_pos)
@@ -293,9 +300,9 @@ class _PreNormMoE(torch.autograd.Function):
     def forward(ctx, x, norm_w, wr, w1, w3, w2, eps, k, bias, shadows, grad_params, add_residual):
         T, H = x.shape
         E = wr.shape[0]
-        x = x.contiguous()
+        x = _dense(x)
         shadows = shadows or (None, None, None)
-        w1b, w3b, w2b = (sh if sh is not None else ops.cast_bf16(w.contiguous())
+        w1b, w3b, w2b = (sh if sh is not None else ops.cast_bf16(_dense(w))
                          for w, sh in zip((w1, w3, w2), shadows))
         wrb = wr.detach().to(torch.bfloat16)
         if norm_w is not None and bias is None and T > 0 and ops.rmsnorm_router_supported(H, E, k):
@@ -343,7 +350,7 @@ class _PreNormMoE(torch.autograd.Function):
         T = ctx.x_shape[0]
         if dout is None:
             dout = torch.zeros(ctx.x_shape, dtype=ctx.x_dtype, device=xn.device)
-        dout = dout.contiguous()
+        dout = _dense(dout)
         if dout.dtype != ctx.x_dtype:
             dout = dout.to(ctx.x_dtype)
         dyp, _ = ops.combine_bwd(dout, None, gates, pos_to_row, k, row_to_pos)
@@ -413,9 +420,9 @@ class _ExpertsRows(torch.autograd.Function):
     def forward(ctx, rows, ids, w1, w3, w2, grad_params):
         R, H = rows.shape
         E = w1.shape[0]
-        rows = rows.contiguous()
-        ids32 = ids.to(torch.int32).contiguous()
-        w1b, w3b, w2b = (ops.cast_bf16(w.contiguous()) for w in (w1, w3, w2))
+        rows = _dense(rows)
+        ids32 = _dense(ids.to(torch.int32))
+        w1b, w3b, w2b = (ops.cast_bf16(_dense(w)) for w in (w1, w3, w2))
         counts, offs, pos_to_row, row_to_pos, bad = ops.histogram_scan(ids32, E, return_bad=True)
         xp = ops.permute_fwd(rows, pos_to_row, 1)
         train = any(ctx.needs_input_grad)
@@ -437,7 +444,7 @@ class _ExpertsRows(torch.autograd.Function):
         if dout is None:
             dout = torch.zeros(ctx.out_shape, dtype=ctx.x_dtype, device=xp.device)
         R = dout.shape[0]
-        dout = dout.contiguous()
+        dout = _dense(dout)
         if dout.dtype not in (torch.bfloat16, torch.float32):
             dout = dout.float()
         dyp, _ = ops.combine_bwd(dout, None, None, pos_to_row, 1)
