@@ -684,3 +684,69 @@ def test_strided_and_unaligned_inputs(P, entry):
     c = run(flat[5:5 + T * H].view(T, H), dy_d)
     for t_a, t_c in zip(a, c):
         assert torch.equal(t_a, t_c)
+
+
+@pytest.mark.parametrize("entry", ENTRIES + ("experts_rows",))
+@pytest.mark.parametrize("I", [64, 256])   # 256: the width at which dW1 and dW3 share one launch
+def test_gradients_for_a_subset_of_the_inputs(P, entry, I):
+    """Frozen experts, a frozen router, an input that needs no gradient: whatever subset asks
+    for gradients gets the bits the full backward pass gives, and the rest gets none."""
+    T, H, E, k = 200, 128, 4, 2
+    dev = "cuda"
+    g = torch.Generator().manual_seed(21)
+    rnd = lambda *s_, std=1.0: (torch.randn(*s_, generator=g) * std).to(torch.bfloat16).to(dev)
+    base = {"x": rnd(T, H), "wr": rnd(E, H, std=0.3), "w1": rnd(E, I, H, std=0.1), "w3": rnd(E, I, H, std=0.1),
+            "w2": rnd(E, H, I, std=0.1)}
+    dy = rnd(T, H)
+    ids = torch.randint(0, E, (T,), generator=g).to(dev)
+    names = ("x", "wr", "w1", "w3", "w2") if entry != "experts_rows" else ("x", "w1", "w3", "w2")
+
+    def run(wanted):
+        t = {n: base[n].clone().requires_grad_(n in wanted) for n in base}
+        if entry == "moe_ffn":
+            out = P.moe_ffn(t["x"], F.linear(t["x"], t["wr"]), t["w1"], t["w3"], t["w2"], k)
+        elif entry == "routed_moe":
+            out, _ = P.routed_moe(t["x"], t["wr"], t["w1"], t["w3"], t["w2"], k)
+        else:
+            out = P.experts_rows(t["x"], ids, t["w1"], t["w3"], t["w2"])
+        out.backward(dy)
+        return out.detach(), {n: t[n].grad for n in names}
+
+    out_all, full = run(set(names))
+    assert all(v is not None for v in full.values())
+    subsets = [{"x"}, {"w1"}, {"w3"}, {"w2"}, {"w1", "w3"}, {"w1", "w2"}, {"x", "w3"}, set(names) - {"x"}]
+    if "wr" in names:
+        subsets += [{"wr"}, {"x", "wr"}, set(names) - {"wr"}]
+    for wanted in subsets:
+        _say("gradients wanted:", sorted(wanted))
+        out, got = run(wanted)
+        assert torch.equal(out, out_all)
+        for n in names:
+            if n in wanted:
+                assert got[n] is not None and torch.equal(got[n], full[n]), n
+            else:
+                assert got[n] is None, n
+
+
+@pytest.mark.parametrize("entry", ENTRIES + ("experts_rows",))
+def test_backward_twice_through_a_retained_graph(P, entry):
+    """The backward pass leaves what the forward pass saved untouched: a second pass over a
+    retained graph adds the same gradients again (doubling is exact in any float format)."""
+    T, H, I, E, k = 300, 128, 256, 4, 2
+    dev = "cuda"
+    g = torch.Generator().manual_seed(22)
+    rnd = lambda *s_, std=1.0: (torch.randn(*s_, generator=g) * std).to(torch.bfloat16).to(dev).requires_grad_(True)
+    x, wr, w1, w3, w2 = rnd(T, H), rnd(E, H, std=0.3), rnd(E, I, H, std=0.1), rnd(E, I, H, std=0.1), rnd(E, H, I, std=0.1)
+    dy = rnd(T, H).detach()
+    ids = torch.randint(0, E, (T,), generator=g).to(dev)
+    if entry == "moe_ffn":
+        out = P.moe_ffn(x, F.linear(x, wr), w1, w3, w2, k)
+    elif entry == "routed_moe":
+        out, _ = P.routed_moe(x, wr, w1, w3, w2, k)
+    else:
+        out = P.experts_rows(x, ids, w1, w3, w2)
+    out.backward(dy, retain_graph=True)
+    once = [t.grad.clone() for t in (x, w1, w3, w2)]
+    out.backward(dy)
+    for t, o in zip((x, w1, w3, w2), once):
+        assert torch.equal(t.grad, o * 2)

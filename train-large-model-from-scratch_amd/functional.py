@@ -37,6 +37,7 @@ from __future__ import annotations
 import torch
 
 from . import ops
+from .ops import dense as _dense
 
 
 _SPLIT_ROWS = 512  # tokens per partial sum of the router weight gradient
@@ -60,13 +61,6 @@ class _RouterLinear(torch.autograd.Function):
         if ctx.needs_input_grad[1]:
             dw = _router_wgrad(dlogits, x, w.dtype)
         return dx, dw
-
-
-def _dense(t: torch.Tensor) -> torch.Tensor:
-    """Contiguous and 16-byte aligned, as the kernels need their buffers: a copy only for a
-    strided view or a view that starts in the middle of an aligned block."""
-    t = t.contiguous()
-    return t if t.data_ptr() % 16 == 0 else t.clone()
 
 
 def _router_wgrad(dlogits, x, w_dtype):

@@ -29,6 +29,13 @@ def _p(t: torch.Tensor | None):
     return t.data_ptr()
 
 
+def dense(t: torch.Tensor) -> torch.Tensor:
+    """Contiguous and 16-byte aligned, as the kernels need their buffers: a copy only for a
+    strided view or a view that starts in the middle of an aligned block."""
+    t = t.contiguous()
+    return t if t.data_ptr() % 16 == 0 else t.clone()
+
+
 def _stream():
     return torch.cuda.current_stream().cuda_stream
 

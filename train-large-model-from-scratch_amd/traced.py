@@ -38,8 +38,8 @@ def ffn_fwd(x: Tensor, logits: Tensor, w1: Tensor, w3: Tensor, w2: Tensor, k: in
     Without `train` g and u are empty; a weight that already is bf16 has an empty copy."""
     T, H = x.shape
     E = logits.shape[1]
-    x, logits = x.contiguous(), logits.contiguous()
-    wb = [w.contiguous() if w.dtype == _BF16 else ops.cast_bf16(w.contiguous()) for w in (w1, w3, w2)]
+    x, logits = ops.dense(x), ops.dense(logits)
+    wb = [ops.dense(w) if w.dtype == _BF16 else ops.cast_bf16(ops.dense(w)) for w in (w1, w3, w2)]
     ids, gates = ops.router_topk(logits, k, None)
     _, offs, pos_to_row, row_to_pos = ops.histogram_scan(ids, E)
     xp = ops.permute_fwd(x, pos_to_row, k, row_to_pos)
@@ -74,7 +74,7 @@ def ffn_bwd(dout: Tensor, xp: Tensor, g: Tensor, u: Tensor, act: Tensor, gates: 
     T = dout.shape[0]
     E = offs.numel() - 1
     f32 = torch.float32
-    dout = dout.contiguous()
+    dout = ops.dense(dout)
     if dout.dtype not in (_BF16, f32):
         dout = dout.float()
     dyp, _ = ops.combine_bwd(dout, None, gates, pos_to_row, k, row_to_pos)
