@@ -750,3 +750,41 @@ def test_backward_twice_through_a_retained_graph(P, entry):
     out.backward(dy)
     for t, o in zip((x, w1, w3, w2), once):
         assert torch.equal(t.grad, o * 2)
+
+
+def test_module_called_in_fp32_without_autocast(P):
+    """fp32 parameters, fp32 input, no autocast: the router product is the fp32 `nn.Linear`
+    product (fp32 logits, so the selection follows fp32 values), the experts still compute in
+    bf16 on the matrix cores; outputs and every gradient are fp32."""
+    cfg = P.ModelConfig(hidden_size=128, num_experts=8, num_experts_per_tok=2, moe_intermediate_size=64,
+                        init_std=0.05)
+    m = P.MoE(cfg, 2)
+    B, T, H = 2, 100, 128
+    g = torch.Generator().manual_seed(12)
+    x = torch.randn(B, T, H, generator=g).cuda().requires_grad_(True)
+    dy = torch.randn(B, T, H, generator=g).cuda()
+    out, gate_logits = m(x)
+    assert out.dtype == torch.float32 and gate_logits.dtype == torch.float32
+    want_logits = F.linear(x.detach(), m.router.weight.detach())
+    assert torch.allclose(gate_logits, want_logits, atol=1e-5, rtol=1e-5)
+    out.backward(dy)
+    assert all(p.grad is not None and p.grad.dtype == torch.float32 for p in m.parameters())
+    assert x.grad.dtype == torch.float32
+    r = lambda t: t.detach().cpu().to(torch.bfloat16)
+    wr32 = m.router.weight.detach().cpu()
+    w1, w3, w2 = r(m.experts_gate_weights), r(m.experts_up_weights), r(m.experts_down_weights)
+    lg = gate_logits.detach().cpu().reshape(-1, 8)
+    xs = r(x).reshape(-1, H)
+    f = O.moe_forward(xs, wr32, w1, w3, w2, 2, logits=lg)
+    b = O.moe_backward(f, dy.cpu().reshape(-1, H), wr32, w1, w3, w2)
+    fe = O.moe_forward(xs, wr32, w1, w3, w2, 2, logits=lg, emulate_bf16=True)
+    be = O.moe_backward(fe, dy.cpu().reshape(-1, H), wr32, w1, w3, w2, emulate_bf16=True)
+    check("out", out.reshape(-1, H), f["out"], say=_say)
+    for name, t in (("dw1", m.experts_gate_weights.grad), ("dw3", m.experts_up_weights.grad),
+                    ("dw2", m.experts_down_weights.grad)):
+        check(name, t, b[name], be[name], say=_say, klass="wgrad")
+    # the router weight gradient and dx carry the fp32 router path: compared norm-wise
+    for name, t, ref in (("dwr", m.router.weight.grad, b["dwr"]), ("dx", x.grad.reshape(-1, H), b["dx"])):
+        rel = ((t.cpu().float() - ref.float()).norm() / ref.float().norm()).item()
+        _say(f"  {name}: rel_fro {rel:.3e}")
+        assert rel <= 1e-2, name
