@@ -526,6 +526,9 @@ ODD_SHAPES = [
     (1, 64, 32, 4, 2), (7, 72, 40, 3, 3), (50, 128, 64, 1, 1), (33, 256, 136, 16, 16), (5, 64, 64, 32, 4),
     (300, 520, 264, 6, 2), (129, 1024, 8, 8, 1), (1000, 8, 512, 5, 2), (64, 2048, 24, 64, 8),
     (257, 96, 1032, 2, 2), (513, 320, 320, 12, 5), (2, 4096, 16, 4, 4),
+    # more experts than a wavefront has lanes, the largest expert count of the routing kernels,
+    # every expert selected by every token at the largest k
+    (400, 64, 32, 130, 6), (96, 128, 64, 512, 8), (20, 64, 32, 64, 64),
 ]
 
 
