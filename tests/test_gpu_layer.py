@@ -397,6 +397,7 @@ def test_module_weight_copies_follow_the_masters(P):
         return O.moe_forward(r(x).reshape(-1, 128), r(m.router.weight), r(m.experts_gate_weights),
                              r(m.experts_up_weights), r(m.experts_down_weights), 2, logits=lg)["out"]
 
+    saved = {k_: v.detach().clone() for k_, v in m.state_dict().items()}
     o1 = fwd()
     c1 = copies()
     assert len(c1) == 3
@@ -435,6 +436,11 @@ def test_module_weight_copies_follow_the_masters(P):
     check("out without the cache", fwd().reshape(-1, 128), expected(), say=_say)
     m.experts_down_weights.data.mul_(-1.0)
     check("out without the cache, after another .data write", fwd().reshape(-1, 128), expected(), say=_say)
+    # a checkpoint loaded into the live module (trainer.py:266-300): the copies follow
+    m.cache_bf16_weights = True
+    fwd()
+    m.load_state_dict(saved)
+    assert torch.equal(fwd(), o1)
 
 
 def test_weight_gradients_accumulated_into_grad(P):
