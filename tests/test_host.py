@@ -154,3 +154,56 @@ def test_launch_observer_sees_every_entry_point_call():
     assert seen == [("before", "moe_cast_f32_bf16"), ("after", "moe_cast_f32_bf16")] * 2
     L.call("moe_cast_f32_bf16", None, None, 0, None)
     assert len(seen) == 4
+
+
+# pointers an entry point may be handed as null (documented so in the header); every other
+# pointer must be refused with MOE_ERR_NULL before anything is launched
+_OPTIONAL_POINTERS = {
+    "moe_router_topk_fwd": {"bias"},
+    "moe_histogram_scan_checked": {"bad_ids"}, "moe_histogram_scan_static": {"bad_ids"},
+    "moe_permute_bwd": {"addend"},
+    "moe_gemm_dgrad_down_swiglu_bwd_packed": {"dgate_part"},
+    "moe_combine_fwd": {"gates"}, "moe_combine_fwd_residual": {"gates"},
+    "moe_combine_bwd": {"gates"}, "moe_combine_bwd_by_token": {"gates"},
+    "moe_rmsnorm_bwd": {"d2", "dres"},
+}
+
+
+def test_every_required_pointer_is_checked_before_any_launch():
+    """Each entry point, with each of its required pointers null in turn (the others point at
+    host memory, sizes are small and valid): MOE_ERR_NULL comes back, i.e. the argument checks
+    stop the call before a kernel could see the pointer.  Nothing is launched, so this runs
+    without a GPU (and is harmless with one)."""
+    pkg = load_pkg()
+    L = pkg.lib.load()
+    text = open(os.path.join(ROOT, "include", "moe_gfx950.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    text = re.sub(r"//[^\n]*", "", text)
+    host = ctypes.create_string_buffer(1 << 20)
+    base = (ctypes.addressof(host) + 255) & ~255
+    sizes = {"T": 8, "E": 16, "k": 2, "H": 64, "I": 256, "R": 16, "M": 64, "N": 64, "S": 2, "P": 1, "n": 64}
+    checked = 0
+    for name, (res, args) in pkg.lib.SIGNATURES.items():
+        if res is not ctypes.c_int or ctypes.c_void_p not in args:
+            continue
+        params = re.search(r"\b" + name + r"\s*\(([^)]*)\)", text).group(1).replace("\n", " ").split(",")
+        pnames = [re.split(r"[\s\*]+", p.strip())[-1] for p in params]
+        assert len(pnames) == len(args), name
+        optional = _OPTIONAL_POINTERS.get(name, set()) | {"stream"}
+        for null_at, (a, n) in enumerate(zip(args, pnames)):
+            if a is not ctypes.c_void_p or n in optional:
+                continue
+            vals = []
+            for i, (b, m) in enumerate(zip(args, pnames)):
+                if b is ctypes.c_void_p:
+                    vals.append(None if (i == null_at or m == "stream") else base + 4096 * i)
+                elif b is ctypes.c_int64:
+                    vals.append(sizes.get(m, (1 << 20) if "bytes" in m else 8))
+                elif b is ctypes.c_float:
+                    vals.append(1e-6)
+                else:
+                    vals.append(0)
+            rc = getattr(L.cdll, name)(*vals)
+            assert rc == -1, f"{name}: null `{n}` gave {rc}, not MOE_ERR_NULL"
+            checked += 1
+    assert checked > 90
