@@ -207,3 +207,54 @@ def test_every_required_pointer_is_checked_before_any_launch():
             assert rc == -1, f"{name}: null `{n}` gave {rc}, not MOE_ERR_NULL"
             checked += 1
     assert checked > 90
+
+
+def test_sizes_and_dtypes_are_checked_before_any_launch():
+    """Each entry point with each size argument negative and beyond every limit (2^40) in turn,
+    and each dtype code invalid: a negative MOE_ERR_* comes back.  Pointers point at host memory,
+    so this is for a machine without a GPU only (there a check that let a value through could do
+    no harm: the launch itself fails with 'no device')."""
+    if torch.cuda.is_available():
+        pytest.skip("hands host pointers to the entry points: CPU-only check")
+    pkg = load_pkg()
+    L = pkg.lib.load()
+    text = open(os.path.join(ROOT, "include", "moe_gfx950.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    text = re.sub(r"//[^\n]*", "", text)
+    host = ctypes.create_string_buffer(1 << 20)
+    base = (ctypes.addressof(host) + 255) & ~255
+    sizes = {"T": 8, "E": 16, "k": 2, "H": 64, "I": 256, "R": 16, "M": 64, "N": 64, "S": 2, "P": 1, "n": 64}
+    # sizes that have no upper limit by design: a byte count the caller vouches for, an element count
+    unlimited = {"workspace_bytes", "n"}
+    checked = 0
+    for name, (res, args) in pkg.lib.SIGNATURES.items():
+        if res is not ctypes.c_int or ctypes.c_void_p not in args:
+            continue
+        params = re.search(r"\b" + name + r"\s*\(([^)]*)\)", text).group(1).replace("\n", " ").split(",")
+        pnames = [re.split(r"[\s\*]+", p.strip())[-1] for p in params]
+
+        def call(bad_at, bad):
+            vals = []
+            for i, (b, m) in enumerate(zip(args, pnames)):
+                if b is ctypes.c_void_p:
+                    vals.append(None if m == "stream" else base + 4096 * i)
+                elif i == bad_at:
+                    vals.append(bad)
+                elif b is ctypes.c_int64:
+                    vals.append(sizes.get(m, (1 << 20) if "bytes" in m else 8))
+                elif b is ctypes.c_float:
+                    vals.append(1e-6)
+                else:
+                    vals.append(0)
+            return getattr(L.cdll, name)(*vals)
+
+        for i, (a, n) in enumerate(zip(args, pnames)):
+            if a is ctypes.c_int64:
+                assert call(i, -1) < 0, f"{name}: {n} = -1 accepted"
+                if n not in unlimited:
+                    assert call(i, (1 << 40) + 8) < 0, f"{name}: {n} = 2^40 + 8 accepted"
+                checked += 1
+            elif a is ctypes.c_int and "dtype" in n:
+                assert call(i, 7) == -4, f"{name}: dtype code 7 for {n} not refused as MOE_ERR_DTYPE"
+                checked += 1
+    assert checked > 100

@@ -152,6 +152,7 @@ __global__ __launch_bounds__(256) void positions_kernel(const int32_t* __restric
 // ---- row movers ---------------------------------------------------------------------------
 
 constexpr int ROWS_PER_BLOCK = 4;
+constexpr int64_t MAX_ROW_ELEMS = 65536;  // widest row the movers take (H and I <= 65536 throughout)
 
 // xp[pos,:] = bf16(x[pos_to_row[pos]/k,:])
 template <typename XT>
@@ -486,7 +487,7 @@ extern "C" int moe_permute_fwd(const void* x, int x_dtype, const int32_t* pos_to
   MOE_CHECK_PTR(xp);
   if (!pos_to_row) return MOE_ERR_NULL;
   if (R < 0 || H <= 0 || k <= 0 || (H % 8) != 0) return MOE_ERR_SHAPE;
-  if (R > (int64_t)1 << 30) return MOE_ERR_LIMIT;
+  if (R > (int64_t)1 << 30 || H > MAX_ROW_ELEMS || k > MOE_MAX_TOPK) return MOE_ERR_LIMIT;
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid(mover_grid(R, ROWS_PER_BLOCK)), block(256);
   if (x_dtype == MOE_DT_BF16)
@@ -507,7 +508,7 @@ extern "C" int moe_permute_fwd_scatter(const void* x, int x_dtype, const int32_t
   MOE_CHECK_PTR(xp);
   if (!row_to_pos) return MOE_ERR_NULL;
   if (T < 0 || H <= 0 || k <= 0 || (H % 8) != 0) return MOE_ERR_SHAPE;
-  if (T * k > (int64_t)1 << 30) return MOE_ERR_LIMIT;
+  if (k > MOE_MAX_TOPK || T > (int64_t)1 << 30 || T * k > (int64_t)1 << 30 || H > MAX_ROW_ELEMS) return MOE_ERR_LIMIT;
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid(mover_grid(T, ROWS_PER_BLOCK)), block(256);
   if (x_dtype == MOE_DT_BF16)
@@ -531,7 +532,7 @@ static int combine_like(const uint16_t* y, const float* gates, const int32_t* ro
   if (addend && !aligned16(addend)) return MOE_ERR_ALIGN;
   if (!row_to_pos) return MOE_ERR_NULL;
   if (T < 0 || H <= 0 || k <= 0 || (H % 8) != 0) return MOE_ERR_SHAPE;
-  if (T * k > (int64_t)1 << 30) return MOE_ERR_LIMIT;
+  if (k > MOE_MAX_TOPK || T > (int64_t)1 << 30 || T * k > (int64_t)1 << 30 || H > MAX_ROW_ELEMS) return MOE_ERR_LIMIT;
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid(mover_grid(T, ROWS_PER_BLOCK)), block(256);
   if (out_dtype == MOE_DT_BF16 && addend_dtype == MOE_DT_BF16)
@@ -585,7 +586,7 @@ extern "C" int moe_combine_bwd(const void* dy, int dy_dtype, const uint16_t* y, 
   if (!pos_to_row) return MOE_ERR_NULL;
   if ((dgates != nullptr) != (y != nullptr)) return MOE_ERR_NULL;
   if (R < 0 || H <= 0 || k <= 0 || (H % 8) != 0) return MOE_ERR_SHAPE;
-  if (R > (int64_t)1 << 30) return MOE_ERR_LIMIT;
+  if (R > (int64_t)1 << 30 || H > MAX_ROW_ELEMS || k > MOE_MAX_TOPK) return MOE_ERR_LIMIT;
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid(mover_grid(R, 4)), block(256);
   if (dy_dtype == MOE_DT_BF16)
@@ -658,7 +659,7 @@ extern "C" int moe_dgates_from_blocks(const float* part, int64_t P, const float*
   if (R == 0) return 0;
   if (!part || !gates || !row_to_pos || !dgates) return MOE_ERR_NULL;
   if (R < 0 || P <= 0) return MOE_ERR_SHAPE;
-  if (R > (int64_t)1 << 30) return MOE_ERR_LIMIT;
+  if (R > (int64_t)1 << 30 || P > MAX_ROW_ELEMS) return MOE_ERR_LIMIT;
   hipLaunchKernelGGL(dgates_from_blocks_kernel, dim3((unsigned)((R + 255) / 256)), dim3(256), 0,
                      (hipStream_t)stream, part, (int)P, gates, row_to_pos, (int)R, dgates);
   return moe_launch_status();
