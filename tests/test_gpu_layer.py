@@ -535,6 +535,8 @@ ODD_SHAPES = [
     # more experts than a wavefront has lanes, the largest expert count of the routing kernels,
     # every expert selected by every token at the largest k
     (400, 64, 32, 130, 6), (96, 128, 64, 512, 8), (20, 64, 32, 64, 64),
+    # the widest rows the interface takes, either way round
+    (12, 65536, 8, 2, 1), (12, 8, 65536, 2, 2),
 ]
 
 

@@ -1077,7 +1077,7 @@ extern "C" int moe_gemm_dgrad_gateup_packed(const uint16_t* dgu, const uint16_t*
 extern "C" int moe_gemm_wgrad_pair(const uint16_t* dgu, const uint16_t* xp, const int32_t* offs, int64_t E,
                                    int64_t R, int64_t I, int64_t H, void* dw1, void* dw3, int dw_dtype,
                                    int accumulate, void* stream) {
-  if (int rc = check_common(offs, E, R, 2 * I, H)) return rc;
+  if (int rc = check_common(offs, E, R, I, H)) return rc;  // (the stacked result has 2*I <= 131072 rows)
   // a 256-row tile of the stacked result must not straddle the two halves
   if ((I % CfgMain::BM) != 0) return MOE_ERR_SHAPE;
   MOE_CHECK_PTR(dw1); MOE_CHECK_PTR(dw3);
