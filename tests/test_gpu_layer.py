@@ -534,7 +534,7 @@ ODD_SHAPES = [
     (257, 96, 1032, 2, 2), (513, 320, 320, 12, 5), (2, 4096, 16, 4, 4),
     # more experts than a wavefront has lanes, the largest expert count of the routing kernels,
     # every expert selected by every token at the largest k
-    (400, 64, 32, 130, 6), (96, 128, 64, 512, 8), (20, 64, 32, 64, 64),
+    (400, 64, 32, 130, 6), (96, 128, 64, 512, 8), (20, 64, 32, 64, 64), (40, 64, 32, 512, 64),
     # the widest rows the interface takes, either way round
     (12, 65536, 8, 2, 1), (12, 8, 65536, 2, 2),
 ]
