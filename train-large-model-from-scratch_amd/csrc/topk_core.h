@@ -21,15 +21,31 @@ __device__ __forceinline__ uint64_t moe_topk_key(float logit, int expert) {
   return ((uint64_t)moe_orderable(logit) << 32) | (uint64_t)(0xffffffffu - (uint32_t)expert);
 }
 
+// Wave-wide maximum of a 64-bit key, the same value in every lane.  Four exchange steps inside
+// each row of 16 lanes go through the DPP data path of the vector ALU (neighbour, pair, mirrored
+// half row, mirrored row: no LDS, no waits), then the four row maxima are read as scalars.
+template <int CTRL>
+__device__ __forceinline__ uint64_t moe_dpp_max_step(uint64_t v) {
+  const int lo = (int)(uint32_t)v, hi = (int)(uint32_t)(v >> 32);
+  const uint32_t lo2 = (uint32_t)__builtin_amdgcn_update_dpp(0, lo, CTRL, 0xf, 0xf, false);
+  const uint32_t hi2 = (uint32_t)__builtin_amdgcn_update_dpp(0, hi, CTRL, 0xf, 0xf, false);
+  const uint64_t o = ((uint64_t)hi2 << 32) | lo2;
+  return o > v ? o : v;
+}
 __device__ __forceinline__ uint64_t moe_wave_max_u64(uint64_t v) {
+  v = moe_dpp_max_step<0xB1>(v);   // quad_perm [1,0,3,2]: lane ^ 1
+  v = moe_dpp_max_step<0x4E>(v);   // quad_perm [2,3,0,1]: lane ^ 2
+  v = moe_dpp_max_step<0x141>(v);  // row_half_mirror: the other quad of each 8 lanes
+  v = moe_dpp_max_step<0x140>(v);  // row_mirror: the other half of each 16 lanes
+  const int lo = (int)(uint32_t)v, hi = (int)(uint32_t)(v >> 32);
+  uint64_t best = 0;
 #pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) {
-    uint32_t lo = __shfl_xor((uint32_t)v, off, MOE_WAVE);
-    uint32_t hi = __shfl_xor((uint32_t)(v >> 32), off, MOE_WAVE);
-    uint64_t o = ((uint64_t)hi << 32) | lo;
-    v = o > v ? o : v;
+  for (int row = 0; row < MOE_WAVE / 16; ++row) {
+    const uint64_t o = ((uint64_t)(uint32_t)__builtin_amdgcn_readlane(hi, 16 * row) << 32) |
+                       (uint32_t)__builtin_amdgcn_readlane(lo, 16 * row);
+    best = o > best ? o : best;
   }
-  return v;
+  return best;
 }
 __device__ __forceinline__ float moe_wave_sum_f32(float v) {
 #pragma unroll
