@@ -91,6 +91,8 @@ _lib: MoELib | None = None
 def load() -> MoELib:
     """Load the built library.  There is no fallback: a missing library is an error."""
     global _lib
+    if _lib is not None:  # the usual case, without the lock
+        return _lib
     with _lock:
         if _lib is None:
             if not os.path.exists(LIB_PATH):
