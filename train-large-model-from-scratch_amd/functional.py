@@ -118,35 +118,40 @@ def _wgrad_split(E: int, M: int, N: int, device) -> int:
     return max(1, min(8, _compute_units(device) // max(tiles, 1), 1024 // max(E, 1)))
 
 
-def _gemm_wgrad(a, b, offs, E, dtype, out=None):
+def _gemm_wgrad(a, b, offs, E, dtype, out=None, segs=None):
     """dw[e] (+)= a[rows of e]^T b[rows of e], cut along the rows when that fills the chip
     better: the segments are the "experts" of one launch with fp32 results, summed in a fixed
-    order (reproducible)."""
+    order (reproducible).  `segs` (a dict that lives as long as one backward pass) keeps the
+    segment bounds of these `offs` per split, so that the three stacks share them."""
     M, N = a.shape[1], b.shape[1]
     S = _wgrad_split(E, M, N, a.device)
     if S == 1 or a.shape[0] == 0:
         return ops.gemm_wgrad(a, b, offs, E, dtype, out=out)
-    seg_offs = ops.segment_offsets(offs, E, S)
+    seg_offs = None if segs is None else segs.get(S)
+    if seg_offs is None:
+        seg_offs = ops.segment_offsets(offs, E, S)
+        if segs is not None:
+            segs[S] = seg_offs
     part = ops.gemm_wgrad(a, b, seg_offs, E * S, torch.float32).view(E, S, M, N).sum(1)
     if out is None:
         return part.to(dtype)
     return out.add_(part)
 
 
-def _wgrad(a, b, offs, E, wdtype, needed, param):
+def _wgrad(a, b, offs, E, wdtype, needed, param, segs=None):
     """One stack's weight gradient.  With `param` given the result goes into `param.grad`
     (added to it when it exists) and None is returned for autograd."""
     if not needed:
         return None
     if param is None:
-        return _gemm_wgrad(a, b, offs, E, wdtype)
+        return _gemm_wgrad(a, b, offs, E, wdtype, segs=segs)
     held = param.grad
     if held is None:
-        param.grad = _gemm_wgrad(a, b, offs, E, param.dtype)
+        param.grad = _gemm_wgrad(a, b, offs, E, param.dtype, segs=segs)
         return None
     if (held.dtype in (torch.float32, torch.bfloat16) and held.is_contiguous()
             and held.shape == (E, a.shape[1], b.shape[1]) and held.device == a.device):
-        _gemm_wgrad(a, b, offs, E, held.dtype, out=held)
+        _gemm_wgrad(a, b, offs, E, held.dtype, out=held, segs=segs)
         return None
     return _gemm_wgrad(a, b, offs, E, wdtype)  # a .grad the kernel cannot add to: autograd sums
 
@@ -204,9 +209,10 @@ def _expert_backward(dyp, xp, g, u, act, w1b, w3b, w2b, offs, wdtype, need_w=(Tr
     else:
         dg, du = ops.gemm_dgrad_down(dyp, w2b, g, u, offs)
     dxp = ops.gemm_dgrad_gateup(dg, du, w1b, w3b, offs)
-    dw2 = _wgrad(dyp, act, offs, E, wdtype, need_w[2], into[2])
-    dw1 = _wgrad(dg, xp, offs, E, wdtype, need_w[0], into[0])
-    dw3 = _wgrad(du, xp, offs, E, wdtype, need_w[1], into[1])
+    segs = {}
+    dw2 = _wgrad(dyp, act, offs, E, wdtype, need_w[2], into[2], segs)
+    dw1 = _wgrad(dg, xp, offs, E, wdtype, need_w[0], into[0], segs)
+    dw3 = _wgrad(du, xp, offs, E, wdtype, need_w[1], into[1], segs)
     return dxp, dw1, dw3, dw2, part
 
 

@@ -82,9 +82,10 @@ def ffn_bwd(dout: Tensor, xp: Tensor, g: Tensor, u: Tensor, act: Tensor, gates: 
     dgates = ops.dgates_from_blocks(part, gates, row_to_pos)
     dxp = ops.gemm_dgrad_gateup(dg, du, w1b, w3b, offs)
     wdt = f32 if w_is_f32 else _BF16
-    dw2 = _gemm_wgrad(dyp, act, offs, E, wdt)
-    dw1 = _gemm_wgrad(dg, xp, offs, E, wdt)
-    dw3 = _gemm_wgrad(du, xp, offs, E, wdt)
+    segs = {}
+    dw2 = _gemm_wgrad(dyp, act, offs, E, wdt, segs=segs)
+    dw1 = _gemm_wgrad(dg, xp, offs, E, wdt, segs=segs)
+    dw3 = _gemm_wgrad(du, xp, offs, E, wdt, segs=segs)
     dx = ops.permute_bwd(dxp, row_to_pos, T, k, f32 if x_is_f32 else _BF16)
     dlogits = ops.router_topk_bwd(gates, dgates, ids, T, E, k, f32 if logits_is_f32 else _BF16)
     return dx, dlogits, dw1, dw3, dw2
