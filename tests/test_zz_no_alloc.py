@@ -67,3 +67,40 @@ def test_static_scratch_dispatch_equals_the_workspace_entry(pkg, lib):
         L.call("moe_histogram_scan_static", ids.data_ptr(), R, E, counts.data_ptr(), offs.data_ptr(),
                p2r.data_ptr(), r2p.data_ptr(), bad.data_ptr(), torch.cuda.current_stream().cuda_stream)
     assert (counts == -7).all()
+
+
+def test_static_scratch_dispatch_inside_a_captured_graph(pkg, lib):
+    """What the entry point is for: recorded into a HIP graph (where nothing may allocate) and
+    replayed on new contents of the same buffers, with eager work and synchronisations between
+    the replays; every replay against the workspace entry run eagerly on the same ids."""
+    L = lib
+    R, E = 40000, 64
+    rng = np.random.default_rng(8)
+    ids = torch.zeros(R, dtype=torch.int32, device="cuda")
+    outs = _outputs(R, E)
+
+    def record():
+        L.call("moe_histogram_scan_static", ids.data_ptr(), R, E, outs[0].data_ptr(), outs[1].data_ptr(),
+               outs[2].data_ptr(), outs[3].data_ptr(), outs[4].data_ptr(),
+               torch.cuda.current_stream().cuda_stream)
+
+    record()   # once outside the capture: the first call on a device looks the scratch array's address up
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        record()
+    for rep in range(4):
+        new = rng.integers(0, E, size=R).astype(np.int32)
+        new[rng.choice(R, size=rep, replace=False)] = -1 - rep   # rep invalid ids
+        ids.copy_(torch.from_numpy(new))
+        for o in outs:
+            o.fill_(-7)
+        graph.replay()
+        torch.cuda.synchronize()
+        want = _call_workspace(L, ids, E)
+        torch.cuda.synchronize()
+        for a, b, name in zip(outs, want, ("counts", "offs", "pos_to_row", "row_to_pos", "bad_ids")):
+            assert torch.equal(a, b), (rep, name)
+        assert outs[4].item() == rep
+        # unrelated eager work on the same device between replays
+        _ = (torch.randn(1 << 20, device="cuda") * 2).sum().item()
