@@ -47,10 +47,11 @@ STRICT_CEILING = {"act": 0.15, "wgrad": 0.20, "token_sum": 0.30}
 # Largest norm-wise distance allowed between the device and the bf16-emulating oracle (brought to
 # the device's output dtype).  The two round at the same points, so what separates them is fp32
 # summation order, the hardware exp/rcp, and the rare one-ulp flip of a stored intermediate:
-# measured 0.5e-4 to 3.7e-4 on expert weight gradients, up to 9e-4 on the router's, up to 2.9e-3
-# on bf16 activation gradients (where the two entries also differ in where the expert and router
-# contributions to dx are rounded).  This is the sharp check: 10 to 30 times tighter than the bar.
-VS_EMULATION = {"act": 5e-3, "wgrad": 1.5e-3, "token_sum": 3e-3}
+# measured 0.5e-4 to 3.7e-4 on expert weight gradients, up to 9e-4 on the router's, up to 4.9e-4
+# on bf16 activation gradients (each entry against the emulation of its own rounding points:
+# through `moe_ffn` the router path's gradient reaches x as a separate bf16 tensor).  This is the
+# sharp check: 7 to 30 times tighter than the bar.
+VS_EMULATION = {"act": 1.5e-3, "wgrad": 1.5e-3, "token_sum": 3e-3}
 
 
 def klass_of(name: str) -> str:

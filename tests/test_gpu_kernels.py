@@ -288,7 +288,24 @@ GEMM_SHAPES = [
 ]
 
 
-@pytest.mark.parametrize("R,H,I,E,empty", GEMM_SHAPES)
+def _random_gemm_shapes(n, seed):
+    """Seeded random shapes: row counts around the 256-row tile edges, widths that are multiples
+    of 8 only, expert counts from 1 to 24 with a random subset left without rows."""
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(n):
+        E = int(rng.integers(1, 25))
+        R = int(rng.choice([rng.integers(1, 64), rng.integers(200, 330), rng.integers(500, 3000)]))
+        H = int(rng.integers(1, 76)) * 8
+        I = int(rng.integers(1, 76)) * 8
+        empty = tuple(int(e) for e in rng.choice(E, size=int(rng.integers(0, max(1, E // 3) + 1)), replace=False)) if E > 1 else ()
+        if len(empty) == E:
+            empty = empty[1:]
+        out.append((R, H, I, E, tuple(sorted(empty))))
+    return out
+
+
+@pytest.mark.parametrize("R,H,I,E,empty", GEMM_SHAPES + _random_gemm_shapes(12, 2024))
 def test_expert_gemms_forward_backward(ops, R, H, I, E, empty):
     _say("gemm", R, H, I, E, empty)
     xp, w1, w3, w2, starts = _gemm_case(R, H, I, E, seed=R + H, empty=empty)

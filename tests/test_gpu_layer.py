@@ -79,7 +79,7 @@ def _oracle_once(tag, inp, logits_dev, k):
         _, be = _oracle(inp, logits_dev, k, True, emulate=True)
         keep = ("dx", "dw1", "dw3", "dw2", "dwr")
         _oracle_cache[key] = ({n: f[n] for n in ("ids", "counts", "starts", "pos_to_row", "row_to_pos", "gates", "out")},
-                              {n: b[n] for n in keep}, {n: be[n] for n in keep})
+                              {n: b[n] for n in keep}, {n: be[n] for n in keep + ("dx@moe_ffn",)})
     return _oracle_cache[key]
 
 
@@ -93,7 +93,19 @@ def _oracle(inp, logits_dev, k, backward, emulate=False):
     if backward:
         b = O.moe_backward(f, inp["dy"].float(), inp["wr"], inp["w1"], inp["w3"], inp["w2"],
                            emulate_bf16=emulate)
+        if emulate:
+            # Through `moe_ffn` the router product is its own autograd node, as in the reference:
+            # the expert path's and the router path's gradients reach x as two bf16 tensors
+            # that autograd adds (one more rounding each way than inside `routed_moe`).
+            bf = torch.bfloat16
+            two = b["dx_expert"].to(bf).float() + b["dx_router"].to(bf).float()
+            b["dx@moe_ffn"] = (two.to(bf).float() if inp["x"].dtype == bf else b["dx"]).reshape(b["dx"].shape)
     return f, b
+
+
+def _emu(be, name, entry):
+    """The bf16-emulating oracle's tensor for `name` as the given entry rounds it."""
+    return be["dx@moe_ffn"] if (name == "dx" and entry == "moe_ffn") else be[name]
 
 
 @pytest.mark.parametrize("entry", ENTRIES)
@@ -122,7 +134,7 @@ def test_config2_forward_backward_skewed(P, entry):
     _, be = _oracle(inp, logits, s.k, True, emulate=True)
     check("out", out, f["out"], say=_say)
     for name in ("dx", "dw1", "dw3", "dw2", "dwr"):
-        check(name, grads[name], b[name], be[name], say=_say)
+        check(name, grads[name], b[name], _emu(be, name, entry), say=_say)
     # run-to-run determinism of every gradient
     _, _, _, grads2 = _run_layer(P, inp, s.k, backward=True, entry=entry)
     for name in grads:
@@ -141,7 +153,7 @@ def test_config3_full_size_vs_oracle(P, entry):
     _check_routing(rt, f, s.E)
     check("out", out, f["out"], say=_say)
     for name in ("dx", "dw1", "dw3", "dw2", "dwr"):
-        check(name, grads[name], b[name], be[name], say=_say)
+        check(name, grads[name], b[name], _emu(be, name, entry), say=_say)
 
 
 def test_config3_reduced_tokens_vs_oracle(P):
@@ -154,7 +166,7 @@ def test_config3_reduced_tokens_vs_oracle(P):
     _, be = _oracle(inp, logits, s.k, True, emulate=True)
     check("out", out, f["out"], say=_say)
     for name in ("dx", "dw1", "dw3", "dw2", "dwr"):
-        check(name, grads[name], b[name], be[name], say=_say)
+        check(name, grads[name], b[name], _emu(be, name, "moe_ffn"), say=_say)
 
 
 def test_config3_full_size_properties(P):
@@ -540,7 +552,17 @@ ODD_SHAPES = [
 ]
 
 
-@pytest.mark.parametrize("T,H,I,E,k", ODD_SHAPES)
+def _random_layer_shapes(n, seed):
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(n):
+        E = int(rng.integers(1, 40))
+        k = int(rng.integers(1, min(E, 8) + 1))
+        out.append((int(rng.integers(1, 700)), int(rng.integers(1, 48)) * 8, int(rng.integers(1, 48)) * 8, E, k))
+    return out
+
+
+@pytest.mark.parametrize("T,H,I,E,k", ODD_SHAPES + _random_layer_shapes(10, 77))
 def test_odd_shapes_forward_backward(P, T, H, I, E, k):
     """Forward and backward against the oracle on shapes the benchmark configurations do not
     visit; routing bit-exact, floating point to the usual bar."""
@@ -562,7 +584,7 @@ def test_odd_shapes_forward_backward(P, T, H, I, E, k):
             # at the device's storage points.
             check(name + " (vs the bf16-rounding oracle)", gr[name], be[name], say=_say)
             continue
-        check(name, gr[name], b[name], be[name], say=_say)
+        check(name, gr[name], b[name], _emu(be, name, "moe_ffn"), say=_say)
     counts = f["counts"]
     for e in range(E):  # experts without rows: exactly zero weight gradients
         if counts[e] == 0:
@@ -609,7 +631,12 @@ def test_routed_moe_is_router_linear_plus_moe_ffn(P, x_dtype):
     dl = (torch.randn(T, E, generator=g) * 0.1).to(dev).to(torch.bfloat16)
     torch.autograd.backward([o3, lg3], [dy, dl])
     extra = dl.float().cpu() @ inp["wr"].float()
-    check("dx with a logits gradient", x3.grad, b["dx"] + extra, (be["dx"] + extra).to(x_dtype).float(), say=_say)
+    # the device adds the incoming gradient to its own logits gradient in bf16 and multiplies the
+    # sum by the router weight in one bf16 product
+    bf = torch.bfloat16
+    dl_sum = (be["dlogits"].to(bf) + dl.cpu()).float()
+    em_dx = be["dx_expert"] + (dl_sum @ inp["wr"].float()).to(bf).float()
+    check("dx with a logits gradient", x3.grad, b["dx"] + extra, em_dx.to(x_dtype).float(), say=_say)
 
 
 @pytest.mark.parametrize("entry", ENTRIES + ("experts_rows", "module", "module_prenorm"))
