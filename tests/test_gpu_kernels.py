@@ -169,6 +169,44 @@ def test_histogram_scan_bit_exact(ops, case):
     assert np.array_equal(r2p.cpu().numpy(), or2p.astype(np.int32))
 
 
+def test_dispatch_and_routing_on_random_sizes(ops):
+    """Forty seeded random sizes through the integer kernels -- row counts around the 64-lane and
+    256-row block edges, 1 to 512 experts, skewed and uniform draws -- all bit-exact against
+    numpy; and the same number of random routing problems (E up to 512, k up to 64, both logit
+    dtypes, with and without quantised ties)."""
+    rng = np.random.default_rng(4242)
+    for case in range(40):
+        E = int(rng.choice([1, 2, 3, int(rng.integers(4, 65)), int(rng.integers(65, 513))]))
+        R = int(rng.choice([rng.integers(1, 70), rng.integers(250, 262), rng.integers(1000, 40000)]))
+        if rng.random() < 0.5:
+            ids = rng.integers(0, E, size=R)
+        else:
+            ids = rng.choice(E, size=R, p=rng.dirichlet(np.full(E, 0.2)))
+        _say("random dispatch", case, "R", R, "E", E)
+        counts, offs, p2r, r2p = ops.histogram_scan(torch.from_numpy(ids.astype(np.int32)).cuda(), E)
+        oc, ostarts = O.counts_offsets(ids, E)
+        op2r, or2p = O.stable_permutation(ids)
+        assert np.array_equal(counts.cpu().numpy(), oc.astype(np.int32)), (case, R, E)
+        assert np.array_equal(offs.cpu().numpy(), ostarts), (case, R, E)
+        assert np.array_equal(p2r.cpu().numpy(), op2r.astype(np.int32)), (case, R, E)
+        assert np.array_equal(r2p.cpu().numpy(), or2p.astype(np.int32)), (case, R, E)
+    g = torch.Generator().manual_seed(4243)
+    for case in range(40):
+        E = int(rng.choice([1, 2, 5, int(rng.integers(6, 65)), int(rng.integers(65, 513))]))
+        k = int(rng.integers(1, min(E, 64) + 1))
+        T = int(rng.choice([1, 3, int(rng.integers(4, 300)), int(rng.integers(300, 5000))]))
+        dtype = torch.bfloat16 if rng.random() < 0.5 else torch.float32
+        logits = torch.randn(T, E, generator=g)
+        if rng.random() < 0.4:
+            logits = (logits * 2).round() / 2
+        logits = logits.to(dtype)
+        _say("random routing", case, "T", T, "E", E, "k", k, dtype)
+        ids, gates = ops.router_topk(logits.cuda(), k)
+        oid, osel = O.topk_select(logits, k)
+        assert np.array_equal(ids.cpu().numpy().reshape(T, k), oid.astype(np.int32)), (case, T, E, k)
+        assert torch.allclose(gates.cpu().reshape(T, k), O.gates_from_selected(osel), atol=1e-6, rtol=1e-5)
+
+
 def test_histogram_scan_counts_ids_out_of_range(pkg, ops):
     """Expert ids outside [0, E): counted on the device, rows placed with the nearest valid
     expert (the result equals the sort of the clipped ids), nothing read or written out of
