@@ -28,16 +28,16 @@ HBM_PEAK_GBS = 8000.0
 # are in profiles/grouped_gemm_cfg3_pmc.txt.  bench.py cannot run the profiler on itself, so
 # the figures are carried here and refreshed whenever that profile is.
 MEASURED_HBM_BYTES_PER_LAUNCH = {
-    (3, "gemm_gateup_swiglu_fwd"): 4.044e9,
-    (3, "gemm_down_fwd"): 1.855e9,
-    (3, "gemm_dgrad_down_swiglu_bwd"): 2.483e9,
-    (3, "gemm_dgrad_gateup"): 3.743e9,
+    (3, "gemm_gateup_swiglu_fwd"): 4.009e9,
+    (3, "gemm_down_fwd"): 1.829e9,
+    (3, "gemm_dgrad_down_swiglu_bwd"): 2.465e9,
+    (3, "gemm_dgrad_gateup"): 3.771e9,
     (3, "gemm_wgrad_down"): 1.074e9,
-    (3, "gemm_wgrad_gate_and_up_pair"): 2.15e9,   # from the average over both weight-gradient launches
+    (3, "gemm_wgrad_gate_and_up_pair"): 2.23e9,   # from the average over both weight-gradient launches
     # the same kernels under the names of their entry points (as the in-step events see them)
-    (3, "gemm_dgrad_down_swiglu_bwd_packed"): 2.483e9,
-    (3, "gemm_dgrad_gateup_packed"): 3.743e9,
-    (3, "gemm_wgrad_pair"): 2.15e9,
+    (3, "gemm_dgrad_down_swiglu_bwd_packed"): 2.465e9,
+    (3, "gemm_dgrad_gateup_packed"): 3.771e9,
+    (3, "gemm_wgrad_pair"): 2.23e9,
 }
 
 
