@@ -826,3 +826,46 @@ def test_module_called_in_fp32_without_autocast(P):
         rel = ((t.cpu().float() - ref.float()).norm() / ref.float().norm()).item()
         _say(f"  {name}: rel_fro {rel:.3e}")
         assert rel <= 1e-2, name
+
+
+def test_two_host_threads_on_two_streams(P):
+    """The library keeps no state between calls: two host threads, each on its own stream with
+    its own tensors, run forward+backward at the same time and get the bits a single thread
+    gets (the autograd engine itself calls the backward pass from a thread of its own)."""
+    import threading
+    T, H, I, E, k = 700, 256, 128, 8, 2
+    dev = "cuda"
+
+    def make(seed):
+        g = torch.Generator().manual_seed(seed)
+        rnd = lambda *s_, std=1.0: (torch.randn(*s_, generator=g) * std).to(torch.bfloat16).to(dev)
+        return [rnd(T, H), rnd(E, H, std=0.3), rnd(E, I, H, std=0.1), rnd(E, I, H, std=0.1), rnd(E, H, I, std=0.1), rnd(T, H)]
+
+    def run(tensors, stream, out, reps):
+        with torch.cuda.stream(stream):
+            for _ in range(reps):
+                x, wr, w1, w3, w2 = (t.detach().clone().requires_grad_(True) for t in tensors[:5])
+                o, _ = P.routed_moe(x, wr, w1, w3, w2, k)
+                o.backward(tensors[5])
+                res = [o.detach(), x.grad, wr.grad, w1.grad, w3.grad, w2.grad]
+            stream.synchronize()
+        out.append(res)
+
+    sets = [make(31), make(32)]
+    serial = []
+    for ts in sets:
+        got = []
+        run(ts, torch.cuda.current_stream(), got, 1)
+        serial.append(got[0])
+    torch.cuda.synchronize()
+    results = [[], []]
+    threads = [threading.Thread(target=run, args=(sets[i], torch.cuda.Stream(), results[i], 6)) for i in range(2)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    torch.cuda.synchronize()
+    for i in range(2):
+        assert len(results[i]) == 1
+        for a, b in zip(results[i][0], serial[i]):
+            assert torch.equal(a, b)
