@@ -158,6 +158,10 @@ int moe_gemm_dgrad_down_swiglu_bwd_dgate(const uint16_t* dyp, const uint16_t* w2
  * routed order t*k+j; blocks added in ascending order (reproducible). */
 int moe_dgates_from_blocks(const float* dgate_part, int64_t blocks, const float* gates,
                            const int32_t* row_to_pos, int64_t R, float* dgates, void* stream);
+/* The same result from the inverse map (pos_to_row): positions are walked in order, so the
+ * blocks are read coalesced and only the 4-byte results are scattered (mlp.py:166 backward). */
+int moe_dgates_from_blocks_by_pos(const float* dgate_part, int64_t blocks, const float* gates,
+                                  const int32_t* pos_to_row, int64_t R, float* dgates, void* stream);
 /* Backward of gate/up w.r.t. the rows (autograd of mlp.py:154-155): dxp = dg*W1 + du*W3. */
 int moe_gemm_dgrad_gateup(const uint16_t* dg, const uint16_t* du, const uint16_t* w1,
                           const uint16_t* w3, const int32_t* offs, int64_t E, int64_t R,

@@ -459,6 +459,9 @@ def test_gate_gradients_from_the_dgrad_down_kernel(ops, R, H, I, E, empty):
     again = ops.dgates_from_blocks(ops.gemm_dgrad_down(dyp, w2.cuda(), g, u, offs, dgate_blocks=True)[2],
                                    gates.cuda(), perm.cuda()).cpu()
     assert torch.equal(again, dgates)  # reproducible
+    # the walk by position (coalesced block reads, scattered results): the same bits
+    by_pos = ops.dgates_from_blocks(part, gates.cuda(), perm.cuda(), inv.cuda()).cpu()
+    assert torch.equal(by_pos, dgates)
 
 
 @pytest.mark.parametrize("R,H,I,E,empty", [(1000, 256, 256, 5, ()), (3000, 520, 512, 7, (2, 5)), (8192, 1024, 1024, 8, ()),

@@ -261,7 +261,7 @@ class _MoEFFN(torch.autograd.Function):
         dx = ops.permute_bwd(dxp, row_to_pos, T, k, ctx.x_dtype) if ctx.needs_input_grad[0] else None
         dlogits = None
         if ctx.needs_input_grad[1]:
-            dgates = ops.dgates_from_blocks(part, gates, row_to_pos)
+            dgates = ops.dgates_from_blocks(part, gates, row_to_pos, pos_to_row)
             dlogits = ops.router_topk_bwd(gates, dgates, ids, T, E, k, ctx.logits_dtype)
         return dx, dlogits, dw1, dw3, dw2, None, None, None, None
 
@@ -356,7 +356,7 @@ class _PreNormMoE(torch.autograd.Function):
         dyp, _ = ops.combine_bwd(dout, None, gates, pos_to_row, k, row_to_pos)
         dxp, dw1, dw3, dw2, part = _expert_backward(dyp, xp, g, u, act, w1b, w3b, w2b, offs, ctx.w_dtype,
                                                     ctx.needs_input_grad[3:6], ctx.grad_params, True)
-        dgates = ops.dgates_from_blocks(part, gates, row_to_pos)
+        dgates = ops.dgates_from_blocks(part, gates, row_to_pos, pos_to_row)
         dlogits = ops.router_topk_bwd(gates, dgates, ids, T, E, k, torch.bfloat16)
         if dlogits_ext is not None:
             dlogits = dlogits + dlogits_ext.to(dlogits.dtype)

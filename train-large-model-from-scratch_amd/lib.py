@@ -30,6 +30,7 @@ SIGNATURES = {
     "moe_gemm_dgrad_down_swiglu_bwd_dgate": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp,
                                                     _vp, _vp]),
     "moe_dgates_from_blocks": (_int, [_vp, _i64, _vp, _vp, _i64, _vp, _vp]),
+    "moe_dgates_from_blocks_by_pos": (_int, [_vp, _i64, _vp, _vp, _i64, _vp, _vp]),
     "moe_gemm_dgrad_gateup": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp]),
     "moe_gemm_wgrad": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _int, _int, _vp]),
     "moe_gemm_dgrad_down_swiglu_bwd_packed": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _vp]),

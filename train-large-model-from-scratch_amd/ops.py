@@ -152,13 +152,18 @@ def gemm_dgrad_down(dyp, w2, g, u, offs, dgate_blocks: bool = False):
     return dg, du
 
 
-def dgates_from_blocks(part, gates, row_to_pos):
+def dgates_from_blocks(part, gates, row_to_pos, pos_to_row=None):
     """Gate gradients dgates[r] = <dy[token of r], y[row of r]> from the per-row block sums the
-    dgrad-down kernel left (they hold gate * that product)."""
+    dgrad-down kernel left (they hold gate * that product).  With the inverse map also given the
+    blocks are read in position order (coalesced) and the results scattered: the same values."""
     R = gates.numel()
     dgates = torch.empty(R, dtype=torch.float32, device=gates.device)
-    _lib.load().call("moe_dgates_from_blocks", _p(part), part.shape[0], _p(gates),
-                     _p(row_to_pos), R, _p(dgates), _stream())
+    if pos_to_row is not None:
+        _lib.load().call("moe_dgates_from_blocks_by_pos", _p(part), part.shape[0], _p(gates),
+                         _p(pos_to_row), R, _p(dgates), _stream())
+    else:
+        _lib.load().call("moe_dgates_from_blocks", _p(part), part.shape[0], _p(gates),
+                         _p(row_to_pos), R, _p(dgates), _stream())
     return dgates
 
 

@@ -79,7 +79,7 @@ def ffn_bwd(dout: Tensor, xp: Tensor, g: Tensor, u: Tensor, act: Tensor, gates: 
         dout = dout.float()
     dyp, _ = ops.combine_bwd(dout, None, gates, pos_to_row, k, row_to_pos)
     dg, du, part = ops.gemm_dgrad_down(dyp, w2b, g, u, offs, dgate_blocks=True)
-    dgates = ops.dgates_from_blocks(part, gates, row_to_pos)
+    dgates = ops.dgates_from_blocks(part, gates, row_to_pos, pos_to_row)
     dxp = ops.gemm_dgrad_gateup(dg, du, w1b, w3b, offs)
     wdt = f32 if w_is_f32 else _BF16
     segs = {}
