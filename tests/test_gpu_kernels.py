@@ -244,9 +244,19 @@ def test_histogram_scan_counts_ids_out_of_range(pkg, ops):
     assert rt["bad_ids"].item() == 37 and torch.equal(out_bad, out)
 
 
+def _random_mover_shapes(n, seed):
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(n):
+        E = int(rng.integers(1, 70))
+        k = int(rng.integers(1, min(E, 9) + 1))
+        out.append((int(rng.integers(1, 400)), int(rng.choice([rng.integers(1, 40), rng.integers(40, 600)])) * 8, k, E))
+    return out
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("T,H,k,E", [(300, 256, 2, 8), (64, 2048, 8, 64), (5, 8, 1, 3), (33, 1032, 3, 5),
-                                     (17, 4096, 2, 4)])
+                                     (17, 4096, 2, 4)] + _random_mover_shapes(8, 99))
 def test_permute_and_combine(ops, dtype, T, H, k, E):
     _say("permute/combine", dtype, T, H, k, E)
     g = torch.Generator().manual_seed(T + H)
