@@ -227,10 +227,21 @@ def test_prenorm_moe_odd_shapes(pkg, lib, T, H, I, E, k):
         check("d norm weight", nwd.grad, dnw_ref, dnw_e, say=_say)
 
 
+def _random_norm_router_shapes(n, seed):
+    import numpy as np
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(n):
+        E = int(rng.integers(1, 9)) * 16
+        out.append((int(rng.integers(1, 600)), int(rng.integers(1, 129)) * 32, E, int(rng.integers(1, min(E, 64) + 1)),
+                    torch.float32 if rng.random() < 0.5 else torch.bfloat16))
+    return out
+
+
 @pytest.mark.parametrize("T,H,E,k,x_dt", [
     (1, 64, 16, 2, torch.float32), (37, 256, 32, 4, torch.float32), (300, 1024, 64, 8, torch.bfloat16),
     (8192, 2048, 64, 8, torch.float32), (130, 4096, 128, 64, torch.bfloat16), (17, 2048, 48, 3, torch.float32),
-])
+] + _random_norm_router_shapes(8, 5150))
 def test_norm_router_topk_in_one_kernel(pkg, lib, T, H, E, k, x_dt):
     """RMSNorm + router product + top-k in one kernel against the three separate steps: xn and
     rstd are the same bits as the norm kernel's; the logits equal the library product on those
