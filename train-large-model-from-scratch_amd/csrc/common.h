@@ -40,8 +40,7 @@ __device__ __forceinline__ float bf16hi(uint32_t w) {
 struct Row8 {
   float v[8];
 };
-__device__ __forceinline__ Row8 load8(const uint16_t* p) {
-  const u32x4 w = *reinterpret_cast<const u32x4*>(p);
+__device__ __forceinline__ Row8 row8_from_bits(u32x4 w) {  // eight bf16 as fp32
   Row8 r;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -49,6 +48,9 @@ __device__ __forceinline__ Row8 load8(const uint16_t* p) {
     r.v[2 * i + 1] = bf16hi(w[i]);
   }
   return r;
+}
+__device__ __forceinline__ Row8 load8(const uint16_t* p) {
+  return row8_from_bits(*reinterpret_cast<const u32x4*>(p));
 }
 __device__ __forceinline__ Row8 load8(const float* p) {
   const f32x4 a = *reinterpret_cast<const f32x4*>(p);

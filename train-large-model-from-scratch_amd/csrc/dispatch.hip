@@ -161,16 +161,55 @@ __global__ __launch_bounds__(256) void permute_fwd_kernel(const XT* __restrict__
                                                          int R, int H8, int k,
                                                          uint16_t* __restrict__ xp) {
   const int H = H8 * 8;
+  const bool once = (k == 1);  // every source row is read exactly once: streaming loads
+  if constexpr (sizeof(XT) == 2) {
+    // a pure row permutation of rows of up to 4096 elements: all of the block's loads are
+    // requested before the first store, so that eight 16-byte loads per thread are in flight
+    // instead of two
+    if (once && H8 <= 512) {
+      for (long long blk = blockIdx.x; blk * ROWS_PER_BLOCK < R; blk += gridDim.x) {
+        const int row0 = (int)(blk * ROWS_PER_BLOCK);
+        u32x4 v[ROWS_PER_BLOCK][2];
+#pragma unroll
+        for (int rr = 0; rr < ROWS_PER_BLOCK; ++rr) {
+          const int pos = row0 + rr;
+          const int t = pos < R ? pos_to_row[pos] : 0;
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            const int col = (threadIdx.x + j * 256) * 8;
+            if (pos < R && col < H)
+              v[rr][j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(x + (size_t)t * H + col));
+          }
+        }
+#pragma unroll
+        for (int rr = 0; rr < ROWS_PER_BLOCK; ++rr) {
+          const int pos = row0 + rr;
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            const int col = (threadIdx.x + j * 256) * 8;
+            if (pos < R && col < H) store_bits_nt(xp + (size_t)pos * H + col, v[rr][j]);
+          }
+        }
+      }
+      return;
+    }
+  }
   for (long long blk = blockIdx.x; blk * ROWS_PER_BLOCK < R; blk += gridDim.x) {
     const int row0 = (int)(blk * ROWS_PER_BLOCK);
-    for (int c = threadIdx.x; c < ROWS_PER_BLOCK * H8; c += blockDim.x) {
-      const int pos = row0 + c / H8, col = (c % H8) * 8;
-      if (pos < R) {
-        const int t = pos_to_row[pos] / k;
+#pragma unroll
+    for (int rr = 0; rr < ROWS_PER_BLOCK; ++rr) {
+      const int pos = row0 + rr;
+      if (pos >= R) break;
+      const int t = once ? pos_to_row[pos] : pos_to_row[pos] / k;
+      const XT* src = x + (size_t)t * H;
+      uint16_t* dst = xp + (size_t)pos * H;
+      for (int col = threadIdx.x * 8; col < H; col += 256 * 8) {
         if constexpr (sizeof(XT) == 2) {  // bf16 -> bf16: move the bits
-          store_bits_nt(xp + (size_t)pos * H + col, *reinterpret_cast<const u32x4*>(x + (size_t)t * H + col));
+          const u32x4 bits = once ? __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src + col))
+                                  : *reinterpret_cast<const u32x4*>(src + col);
+          store_bits_nt(dst + col, bits);
         } else {
-          store8_nt(xp + (size_t)pos * H + col, load8(x + (size_t)t * H + col));
+          store8_nt(dst + col, load8(src + col));
         }
       }
     }
@@ -289,9 +328,40 @@ __global__ __launch_bounds__(256) void combine_bwd_kernel(const DT* __restrict__
     const int r = pos_to_row[pos];
     const int t = r / k;
     const float gt = gates ? gates[r] : 1.f;
+    if constexpr (sizeof(DT) == 2) {
+      // the scaled copy alone, rows of up to 4096 elements: the row's loads are all requested
+      // before its first store (eight in flight per lane instead of one)
+      if (!y && H8 <= 8 * MOE_WAVE) {
+        u32x4 v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int c = lane + j * MOE_WAVE;
+          if (c < H8) {
+            const u32x4* src = reinterpret_cast<const u32x4*>(dy + (size_t)t * H + c * 8);
+            v[j] = (k == 1) ? __builtin_nontemporal_load(src) : *src;
+          }
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int c = lane + j * MOE_WAVE;
+          if (c < H8) {
+            Row8 d = row8_from_bits(v[j]);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) d.v[i] *= gt;
+            store8_nt(dyp + (size_t)pos * H + c * 8, d);
+          }
+        }
+        continue;
+      }
+    }
     float dot = 0.f;
     for (int c = lane; c < H8; c += MOE_WAVE) {
-      Row8 d = load8(dy + (size_t)t * H + c * 8);
+      Row8 d;
+      if constexpr (sizeof(DT) == 2) {  // k == 1: every row of dy is read exactly once
+        d = (k == 1) ? load8_nt(dy + (size_t)t * H + c * 8) : load8(dy + (size_t)t * H + c * 8);
+      } else {
+        d = load8(dy + (size_t)t * H + c * 8);
+      }
       if (y) {
         const Row8 yv = load8_nt(y + (size_t)pos * H + c * 8);
 #pragma unroll
