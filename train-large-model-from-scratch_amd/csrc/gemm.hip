@@ -58,10 +58,9 @@ struct GemmArgs {
   int m_split;  // WGRAD: rows m >= m_split of an expert's result go to C1 (as its rows m - m_split); 0: all to C0
 };
 
-template <int BM_, int BN_, int BK_, int WM_, int WN_, int NSET_>
+template <int BM_, int BN_, int BK_, int WM_, int WN_>
 struct TileCfg {
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_;
-  static constexpr int NSET = NSET_;  // register sets carrying k-tiles from HBM to LDS
   static constexpr int NT = WM * WN * MOE_WAVE;
   static constexpr int WTM = BM / WM, WTN = BN / WN;
   static constexpr int FM = WTM / 32, FN = WTN / 32;
@@ -71,16 +70,6 @@ struct TileCfg {
   static constexpr int WAVES_PER_SIMD = NT / 256 * WGS_PER_CU;
   static_assert(WTM % 32 == 0 && WTN % 32 == 0 && BK % 32 == 0, "tile shape");
 };
-
-template <int... Is, typename F>
-__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, Is...>, F&& f) {
-  (f(std::integral_constant<int, Is>{}), ...);
-}
-// f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>), unrolled at compile time
-template <int N, typename F>
-__device__ __forceinline__ void static_for(F&& f) {
-  static_for_impl(std::make_integer_sequence<int, N>{}, f);
-}
 
 // sigmoid from the two hardware transcendentals (v_exp_f32, v_rcp_f32; about 1 ulp each):
 // the epilogues are VALU-bound, and an IEEE division would triple their cost.
@@ -418,16 +407,14 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WAVES_PER_SIMD) void grouped_gemm_ker
   } else {
     opB.init(ldb);
   }
-  // Registers that carry k-tiles from HBM to LDS.  There are NSET sets; k-tile t of an
-  // output tile travels in set t % NSET and is requested NSET iterations before it is
-  // written to LDS, which is what hides the latency of a load that misses L2.
-  constexpr int NSET = Cfg::NSET;
+  // One set of registers carries a k-tile from HBM to LDS: it is requested one iteration
+  // before it is written to LDS, which is what hides the latency of a load that misses L2.
   constexpr int CHA = StA::CH, CHB = DUAL ? StBh::CH : StB::CH;
   constexpr int NCH = CHA + (DUAL ? 2 : 1) * CHB;  // 16-byte chunks per thread per k-tile
   struct Stage {
     u32x4 v[NCH];
   };
-  Stage stg[NSET];
+  Stage stg;
   struct TileSrc {
     __amdgpu_buffer_rsrc_t a, b0, b1;
     int k_left;
@@ -486,23 +473,6 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WAVES_PER_SIMD) void grouped_gemm_ker
     for (int c = 0; c < NCH; ++c) store_chunk(c, st, buf);
   };
   using std::integral_constant;
-  // run f(integral_constant<int, s>) for the set index s known only at run time (uniform)
-  auto with_set = [&](int s, auto&& f) {
-    if constexpr (NSET == 1) f(integral_constant<int, 0>{});
-    else if constexpr (NSET == 2) { if (s == 0) f(integral_constant<int, 0>{}); else f(integral_constant<int, 1>{}); }
-    else if constexpr (NSET == 3) {
-      if (s == 0) f(integral_constant<int, 0>{});
-      else if (s == 1) f(integral_constant<int, 1>{});
-      else f(integral_constant<int, 2>{});
-    } else {
-      static_assert(NSET == 4, "1..4 register sets");
-      if (s == 0) f(integral_constant<int, 0>{});
-      else if (s == 1) f(integral_constant<int, 1>{});
-      else if (s == 2) f(integral_constant<int, 2>{});
-      else f(integral_constant<int, 3>{});
-    }
-  };
-
   const int a_off = StA::lane_off(lane), b_off = StB::lane_off(lane);
   // LDS row of column-fragment jn for this wave
   auto bfrag_row = [&](int jn) {
@@ -553,10 +523,10 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WAVES_PER_SIMD) void grouped_gemm_ker
   //                   tile kt+2 requested | fragments of step s+1 read
   //   last phase      barrier (stage kt fully read, stage kt+1 fully written) | MFMAs of the
   //                   last step | first fragment reads of stage kt+1 hide behind them
-  auto body = [&](auto par_c, auto set_c, const Tile& t, int kt) {
+  auto body = [&](auto par_c, const Tile& t, int kt) {
     constexpr int buf = decltype(par_c)::value;  // LDS stage of k-tile kt == parity of kt
-    Stage& st = stg[decltype(set_c)::value];     // holds k-tile kt+1, refilled with kt+1+NSET
-    const TileSrc ts = tile_src(t, kt + 1 + NSET);
+    Stage& st = stg;                             // holds k-tile kt+1, refilled with kt+2
+    const TileSrc ts = tile_src(t, kt + 2);
     constexpr int NSLOT = (KS - 1) * NMMA;  // MFMA slots before the barrier
 #pragma unroll
     for (int ks = 0; ks < KS - 1; ++ks) {
@@ -610,7 +580,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WAVES_PER_SIMD) void grouped_gemm_ker
   // k-tile on into LDS at the end of that epilogue was measured 3 % slower)
   constexpr bool EARLY_REQUEST = (MODE != DGRAD_DOWN);
   constexpr int HALF_WAVES = Cfg::WM * Cfg::WN / 2;
-  constexpr bool STAGE_EARLY = EARLY_REQUEST && NSET == 1 &&
+  constexpr bool STAGE_EARLY = EARLY_REQUEST &&
                                NSTRIP * SBYTES * HALF_WAVES <= StA::LDS_ELEMS * 2 &&
                                NSTRIP * SBYTES * HALF_WAVES <= StB::LDS_ELEMS * 2;
   static_assert(NSTRIP * SBYTES * Cfg::WM * Cfg::WN <= lds_bytes<MODE, Cfg>(), "strips fit in the stages");
@@ -794,16 +764,11 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WAVES_PER_SIMD) void grouped_gemm_ker
   };
 
   // ---- the tile loop
-  // At the top of the loop the first min(NSET, nkt) k-tiles of `cur` are already on their
-  // way into the register sets (requested before the previous tile's epilogue).
+  // At the top of the loop the first k-tile of `cur` is already on its way into the staging
+  // registers (requested before the previous tile's epilogue).
   auto request_first = [&](const Tile& t) {
-    static_for<NSET>([&](auto sc) {
-      constexpr int s = decltype(sc)::value;
-      if (s < t.nkt) load_tile(t, s, stg[s]);
-    });
+    if (0 < t.nkt) load_tile(t, 0, stg);
   };
-  constexpr int PERIOD = (NSET % 2 == 0) ? NSET : 2 * NSET;  // lcm(2, NSET), at least 2
-  constexpr int UNROLL = PERIOD < 2 ? 2 : PERIOD;
   Tile cur;
   if (t_next >= t_hi || !locate(t_next, cur)) return;
   request_first(cur);
@@ -825,8 +790,8 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WAVES_PER_SIMD) void grouped_gemm_ker
     const int nkt = cur.nkt;
     if (nkt > 0) {
       if (!staged) {
-        store_tile(stg[0], 0);
-        if (NSET < nkt) load_tile(cur, NSET, stg[0]);
+        store_tile(stg, 0);
+        if (1 < nkt) load_tile(cur, 1, stg);
         lds_barrier();
       }
       if (!idle) f_read_all(0, 0, fr[0]);
@@ -834,36 +799,30 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WAVES_PER_SIMD) void grouped_gemm_ker
     int kt = 0;
     if (idle) {
       for (; kt < nkt; ++kt) {
-        const bool has1 = kt + 1 < nkt, hasn = kt + 1 + NSET < nkt;
+        const bool has1 = kt + 1 < nkt, has2 = kt + 2 < nkt;
         if (has1) {
-          with_set((kt + 1) % NSET, [&](auto sc) {
-            store_tile(stg[decltype(sc)::value], (kt & 1) ^ 1);
-            if (hasn) load_tile(cur, kt + 1 + NSET, stg[decltype(sc)::value]);
-          });
+          store_tile(stg, (kt & 1) ^ 1);
+          if (has2) load_tile(cur, kt + 2, stg);
           lds_barrier();
         }
       }
     }
-    // steady iterations: k-tile kt+1+NSET exists and nothing needs masking
-    const int steady_end = cur.need_mask ? 0 : nkt - 1 - NSET;
-    for (; kt + UNROLL - 1 < steady_end; kt += UNROLL) {
-      static_for<UNROLL>([&](auto uc) {
-        constexpr int u = decltype(uc)::value;
-        body(integral_constant<int, u % 2>{}, integral_constant<int, (u + 1) % NSET>{}, cur, kt + u);
-      });
+    // steady iterations (two at a time: the stage index is a compile-time constant): k-tile
+    // kt+2 exists and nothing needs masking
+    const int steady_end = cur.need_mask ? 0 : nkt - 2;
+    for (; kt + 1 < steady_end; kt += 2) {
+      body(integral_constant<int, 0>{}, cur, kt);
+      body(integral_constant<int, 1>{}, cur, kt + 1);
     }
     for (; kt < nkt; ++kt) {  // last iterations (and every iteration when masking): same
       const int buf = kt & 1;  // order of events, conditions evaluated, no static schedule
-      const bool has1 = kt + 1 < nkt, hasn = kt + 1 + NSET < nkt;
-      const int set = (kt + 1) % NSET;
+      const bool has1 = kt + 1 < nkt, has2 = kt + 2 < nkt;
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         if (ks + 1 < KS) f_read_all(buf, ks + 1, fr[(ks + 1) & 1]);
         if (ks == 0 && has1) {
-          with_set(set, [&](auto sc) {
-            store_tile(stg[decltype(sc)::value], buf ^ 1);
-            if (hasn) load_tile(cur, kt + 1 + NSET, stg[decltype(sc)::value]);
-          });
+          store_tile(stg, buf ^ 1);
+          if (has2) load_tile(cur, kt + 2, stg);
         }
         if (ks == KS - 1 && has1) {
           lds_barrier();
@@ -883,8 +842,8 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WAVES_PER_SIMD) void grouped_gemm_ker
     auto stage_next = [&]() {
       if constexpr (STAGE_EARLY) {
         if (more && nxt.nkt > 0) {
-          store_tile(stg[0], 0);
-          if (1 < nxt.nkt) load_tile(nxt, 1, stg[0]);
+          store_tile(stg, 0);
+          if (1 < nxt.nkt) load_tile(nxt, 1, stg);
           staged = true;
         }
       }
@@ -914,10 +873,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WAVES_PER_SIMD) void grouped_gemm_ker
 #define MOE_WM 2
 #define MOE_WN 4
 #endif
-#ifndef MOE_NSET
-#define MOE_NSET 1
-#endif
-using CfgMain = TileCfg<MOE_BM, MOE_BN, MOE_BK, MOE_WM, MOE_WN, MOE_NSET>;
+using CfgMain = TileCfg<MOE_BM, MOE_BN, MOE_BK, MOE_WM, MOE_WN>;
 
 int compute_units() {
   static int cus = 0;  // same answer from every thread; a benign race at worst repeats the query
