@@ -14,8 +14,11 @@
  *     stay valid until the work enqueued on `stream` has run.  bf16 is passed as
  *     `uint16_t` storage.  `dtype` arguments: MOE_DT_BF16 or MOE_DT_F32.
  *   - Every call only enqueues kernels on `stream` (a hipStream_t passed as void*); it
- *     never synchronises, allocates, prints or throws, and keeps no state between calls,
- *     so it may be called from any host thread.
+ *     never synchronises, allocates, prints or throws, so it may be called from any host
+ *     thread.  What the library keeps between calls is a few facts per GPU that it asks the
+ *     runtime for once (the compute-unit count, "this kernel's shared-memory attribute is
+ *     set", the address of the fixed scratch array of moe_histogram_scan_static), looked up
+ *     by the device that is current at the call; no result depends on an earlier call.
  *   - Return value: 0 on success; a positive hipError_t if a launch failed; a negative
  *     MOE_ERR_* code if an argument check failed (nothing is enqueued then).
  *   - Alignment: H and I must be multiples of 8 (rows are moved as 16-byte vectors) and
@@ -91,12 +94,18 @@ int moe_histogram_scan_checked(const int32_t* ids, int64_t R, int64_t E, int32_t
  * point of the call (code under HIP graph capture, serving loops with a frozen memory plan,
  * harnesses that forbid hipMalloc).  The per-wave histograms go to a fixed array of
  * moe_static_scratch_bytes() (4 MiB) that the library holds in every GPU's memory until the
- * process ends; MOE_ERR_WORKSPACE if moe_dispatch_workspace_bytes(R, E) exceeds it (i.e.
- * ceil(R/256) * (E+1) * 4 > 4 MiB: up to 1 M routed rows at 512 experts, 16 M at 64).  All calls
- * on one GPU share that array: two such calls that overlap in time on one GPU (different
- * streams, or graphs replayed concurrently) race; calls ordered on one stream do not.  Results
- * are bit-identical to moe_histogram_scan_checked. */
+ * process ends; MOE_ERR_WORKSPACE if moe_dispatch_workspace_bytes(R, E) exceeds it, i.e. if
+ * R > moe_static_scratch_max_rows(E) = floor(4 MiB / (4 * (E+1))) * 256: 523 264 routed rows at
+ * 512 experts, 4 129 536 at 64, 29 826 048 at 8.
+ * RACE: all calls on one GPU share that one array.  Two such calls that overlap in time on one GPU
+ * (different streams, host threads whose streams are not ordered, graphs replayed concurrently)
+ * overwrite each other's histograms and return wrong permutations WITHOUT an error code; calls
+ * ordered on one stream do not.  moe_static_scratch_bytes() is also the set-up call: it looks the
+ * array's address up on the current device, so a caller that asks for the size before it starts
+ * capturing a graph leaves no runtime query for the first moe_histogram_scan_static.  Results are
+ * bit-identical to moe_histogram_scan_checked. */
 int64_t moe_static_scratch_bytes(void);
+int64_t moe_static_scratch_max_rows(int64_t E);
 int moe_histogram_scan_static(const int32_t* ids, int64_t R, int64_t E, int32_t* counts,
                               int32_t* offs, int32_t* pos_to_row, int32_t* row_to_pos,
                               int32_t* bad_ids, void* stream);

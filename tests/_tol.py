@@ -56,7 +56,7 @@ VS_EMULATION = {"act": 1.5e-3, "wgrad": 1.5e-3, "token_sum": 3e-3}
 
 def klass_of(name: str) -> str:
     n = name.lower()
-    if "dwr" in n or "router" in n or "dlogits" in n or "dgates" in n or "d norm" in n:
+    if "dwr" in n or "router" in n or "dlogits" in n or "dgates" in n or "d norm" in n or "dbias" in n:
         return "token_sum"
     if "dw" in n or ".grad" in n or "weights" in n:
         return "wgrad"

@@ -49,7 +49,7 @@ def _run_layer(P, inp, k, backward, dy_from_out=False, entry="moe_ffn"):
     wr = inp["wr"].to(dev).requires_grad_(backward)
     ws = [inp[n].to(dev).requires_grad_(backward) for n in ("w1", "w3", "w2")]
     bias = inp.get("bias")
-    bias = None if bias is None else bias.to(dev)
+    bias = None if bias is None else bias.to(dev).requires_grad_(backward)
     if entry == "moe_ffn":
         logits = F.linear(x, wr)
         out, rt = P.moe_ffn(x, logits, *ws, k, bias=bias, return_routing=True)
@@ -63,6 +63,8 @@ def _run_layer(P, inp, k, backward, dy_from_out=False, entry="moe_ffn"):
         dy = dy.to(out.dtype)
         out.backward(dy)
         grads = {"dy": dy, "dx": x.grad, "dwr": wr.grad, "dw1": ws[0].grad, "dw3": ws[1].grad, "dw2": ws[2].grad}
+        if bias is not None:
+            grads["dbias"] = bias.grad
     return out.detach(), logits.detach(), rt, grads
 
 
@@ -135,6 +137,10 @@ def test_config2_forward_backward_skewed(P, entry):
     check("out", out, f["out"], say=_say)
     for name in ("dx", "dw1", "dw3", "dw2", "dwr"):
         check(name, grads[name], b[name], _emu(be, name, entry), say=_say)
+    # the router bias is an input like any other: its gradient (fp32 [E], the column sum of the
+    # logits' gradient) against the oracle's
+    assert grads["dbias"].dtype == torch.float32 and grads["dbias"].shape == (s.E,)
+    check("dbias", grads["dbias"], b["dbias"], be["dbias"], say=_say)
     # run-to-run determinism of every gradient
     _, _, _, grads2 = _run_layer(P, inp, s.k, backward=True, entry=entry)
     for name in grads:
@@ -347,6 +353,43 @@ def test_module_under_autocast_matches_oracle(P):
     mb = P.MoE(cfg, 2).to(torch.bfloat16)
     o2, l2 = mb(x.detach().to(torch.bfloat16))
     assert o2.dtype == torch.bfloat16 and l2.dtype == torch.bfloat16
+
+
+def test_router_hooks_fire_and_prenorm_router_switch(P):
+    """Hooks registered on `moe.router` (an `nn.Linear`, mlp.py:65) run as they would in the
+    reference, with the same results as without them; and `fused_router = False` makes the
+    pre-norm entry select on the library product's logits, bit-equal to `forward`'s."""
+    _say("router hooks; fused_router switch")
+    cfg = P.ModelConfig(hidden_size=256, num_experts=16, num_experts_per_tok=2, moe_intermediate_size=64,
+                        init_std=0.05)
+    m = P.MoE(cfg, 2)
+    x = torch.randn(2, 96, 256, generator=torch.Generator().manual_seed(5)).cuda()
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        out0, lg0 = m(x)
+    seen = []
+    h = m.router.register_forward_hook(lambda mod, inp, out: seen.append(out.detach().clone()))
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        out1, lg1 = m(x)
+    assert len(seen) == 1 and torch.equal(seen[0], lg1)
+    assert torch.equal(lg0, lg1) and torch.equal(out0, out1)
+    norm = torch.nn.Module()
+    norm.weight = torch.nn.Parameter(torch.ones(256, device="cuda"))
+    norm.variance_epsilon = 1e-6
+    norm.forward = lambda t: (t.float() * torch.rsqrt(t.float().pow(2).mean(-1, keepdim=True) + 1e-6)).to(t.dtype) * norm.weight
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        m.forward_prenorm(x, norm)
+    assert len(seen) == 2   # the pre-norm entry falls back to the module's own call of the router
+    h.remove()
+    # fused_router = False: logits are the library product of the normalised bf16 rows
+    m.fused_router = False
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        _, lg_lib = m.forward_prenorm(x, norm)
+    xn, _ = P.ops.rmsnorm_fwd(x.reshape(-1, 256), norm.weight.detach().float(), 1e-6)
+    assert torch.equal(lg_lib.reshape(-1, 16), xn @ m.router.weight.detach().to(torch.bfloat16).t())
+    m.fused_router = True
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        _, lg_fused = m.forward_prenorm(x, norm)
+    assert (lg_fused.float() - lg_lib.float()).abs().max() <= 2 ** -7 * lg_lib.float().abs().max()
 
 
 def test_router_linear_matches_linear(P):

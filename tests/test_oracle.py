@@ -236,6 +236,32 @@ def test_manual_backward_matches_autograd(T, H, E, I, k):
     assert torch.allclose(b["dx_expert"], leaves[0].grad, atol=1e-9)
 
 
+def test_bias_gradient_is_the_column_sum_of_dlogits_by_finite_differences():
+    """`moe_backward()["dbias"]`: the per-expert router bias enters as logit + bias, so its
+    gradient must equal d<dy, out>/d bias, taken here by central differences in fp64 (routing
+    frozen by the margin between the k-th and (k+1)-th logit being far above the step)."""
+    T, H, E, I, k = 12, 16, 6, 8, 2
+    x, wr, w1, w3, w2 = (t.double() for t in _mk(T, H, E, I, seed=77))
+    bias = torch.randn(E, dtype=torch.float64, generator=torch.Generator().manual_seed(3)) * 0.5
+    dy = torch.randn(T, H, dtype=torch.float64, generator=torch.Generator().manual_seed(4))
+    f = O.moe_forward(x, wr, w1, w3, w2, k, bias=bias, compute_dtype=torch.float64)
+    b = O.moe_backward(f, dy, wr, w1, w3, w2)
+    srt = torch.sort(F.linear(x, wr) + bias, dim=-1, descending=True).values
+    assert (srt[:, k - 1] - srt[:, k]).min() > 1e-3
+    h = 1e-6
+    for e in range(E):
+        d = torch.zeros(E, dtype=torch.float64)
+        d[e] = h
+        fp = O.moe_forward(x, wr, w1, w3, w2, k, bias=bias + d, compute_dtype=torch.float64)
+        fm = O.moe_forward(x, wr, w1, w3, w2, k, bias=bias - d, compute_dtype=torch.float64)
+        assert np.array_equal(fp["ids"], f["ids"]) and np.array_equal(fm["ids"], f["ids"])
+        fd = ((fp["out"] - fm["out"]) * dy).sum().item() / (2 * h)
+        assert abs(fd - b["dbias"][e].item()) <= 1e-6 * max(1.0, abs(fd)), (e, fd, b["dbias"][e].item())
+    # and it is not trivially zero, nor is any bias without effect
+    assert b["dbias"].abs().min() > 1e-4
+    assert abs(b["dbias"].sum().item()) < 1e-9   # the softmax over the selected logits is shift-invariant
+
+
 def test_gradcheck_fp64_tiny():
     T, H, E, I, k = 6, 8, 4, 8, 2
     x, wr, w1, w3, w2 = (t.double() for t in _mk(T, H, E, I, seed=40, std=0.5))

@@ -58,9 +58,32 @@ def test_static_scratch_dispatch_equals_the_workspace_entry(pkg, lib):
             assert torch.equal(a, b), (R, E, name)
         assert got[4].item() == (3 if R >= 300 else 0)
         assert got[1][-1].item() == R
-    # beyond the fixed scratch: refused, nothing enqueued
-    R, E = 300 * 256 * 8, 512   # ceil(R/256) * (E+1) * 4 bytes > 4 MiB
-    assert L.cdll.moe_dispatch_workspace_bytes(R, E) > L.cdll.moe_static_scratch_bytes()
+        # and against numpy, not only against the library's other entry: counts, offsets, the
+        # stable sort by expert and its inverse (ids outside [0, E) go with the nearest expert)
+        clipped = np.clip(ids_np, 0, E - 1)
+        np_counts = np.bincount(clipped, minlength=E)
+        np_p2r = np.argsort(clipped, kind="stable")
+        assert np.array_equal(got[0].cpu().numpy(), np_counts), (R, E)
+        assert np.array_equal(got[1].cpu().numpy(), np.concatenate([[0], np.cumsum(np_counts)])), (R, E)
+        assert np.array_equal(got[2].cpu().numpy(), np_p2r), (R, E)
+        inv = np.empty(R, dtype=np.int64)
+        inv[np_p2r] = np.arange(R)
+        assert np.array_equal(got[3].cpu().numpy(), inv), (R, E)
+    # the documented limit, from both sides: the largest size that fits is accepted (and right),
+    # one row more is refused with nothing enqueued
+    E = 512
+    R_max = L.cdll.moe_static_scratch_max_rows(E)
+    assert R_max == (4 << 20) // (4 * (E + 1)) * 256 == 523264
+    assert L.cdll.moe_static_scratch_max_rows(64) == 4129536
+    assert L.cdll.moe_dispatch_workspace_bytes(R_max, E) <= L.cdll.moe_static_scratch_bytes()
+    assert L.cdll.moe_dispatch_workspace_bytes(R_max + 1, E) > L.cdll.moe_static_scratch_bytes()
+    ids_np = rng.integers(0, E, size=R_max)
+    ids = torch.from_numpy(ids_np.astype(np.int32)).cuda()
+    got = _call_static(L, ids, E)
+    torch.cuda.synchronize()
+    assert np.array_equal(got[0].cpu().numpy(), np.bincount(ids_np, minlength=E))
+    assert np.array_equal(got[2].cpu().numpy(), np.argsort(ids_np, kind="stable"))
+    R = R_max + 1
     ids = torch.zeros(R, dtype=torch.int32, device="cuda")
     counts, offs, p2r, r2p, bad = _outputs(R, E)
     with pytest.raises(pkg.lib.MoELibError, match="MOE_ERR_WORKSPACE"):
@@ -84,7 +107,10 @@ def test_static_scratch_dispatch_inside_a_captured_graph(pkg, lib):
                outs[2].data_ptr(), outs[3].data_ptr(), outs[4].data_ptr(),
                torch.cuda.current_stream().cuda_stream)
 
-    record()   # once outside the capture: the first call on a device looks the scratch array's address up
+    # the set-up call (it looks the scratch array's address up on this device), so that the first
+    # call of the entry point may be the captured one
+    assert L.cdll.moe_static_scratch_bytes() == 4 << 20
+    _call_workspace(L, ids, E)   # (the kernels' code is loaded by an eager launch, not under capture)
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):

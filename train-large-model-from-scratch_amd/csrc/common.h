@@ -130,6 +130,16 @@ static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t
     if (!aligned16(p)) return MOE_ERR_ALIGN; \
   } while (0)
 
+// Facts the host side learns once per GPU and keeps (a compute-unit count, "this kernel's
+// attribute is set"): one slot per device id; the caller's current device picks the slot.  Racing
+// first calls at worst repeat an idempotent runtime query.
+constexpr int MOE_MAX_DEVICES = 64;
+static inline int moe_current_device() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MOE_MAX_DEVICES) dev = 0;
+  return dev;
+}
+
 static inline int moe_launch_status() {
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? 0 : (int)e;

@@ -511,7 +511,7 @@ static __device__ __align__(256) unsigned char scratch[MOE_STATIC_SCRATCH_BYTES]
 
 namespace {
 
-constexpr int MAX_DEVICES = 64;
+constexpr int MAX_DEVICES = MOE_MAX_DEVICES;
 void* scratch_of_device[MAX_DEVICES];  // device address of `scratch` on each GPU, 0 = not asked yet
 std::mutex scratch_mutex;
 
@@ -535,7 +535,23 @@ int static_scratch(void** out) {
 
 }  // namespace
 
-extern "C" int64_t moe_static_scratch_bytes(void) { return MOE_STATIC_SCRATCH_BYTES; }
+// Also the set-up call: it looks up the array's address on the current device, so that a caller
+// who asks for the size before capturing a graph (or before entering a region that must not
+// touch the runtime's symbol tables) leaves nothing for the first moe_histogram_scan_static to do.
+extern "C" int64_t moe_static_scratch_bytes(void) {
+  void* ptr = nullptr;
+  (void)static_scratch(&ptr);
+  return MOE_STATIC_SCRATCH_BYTES;
+}
+
+extern "C" int64_t moe_static_scratch_max_rows(int64_t E) {
+  if (E <= 0 || E > MOE_MAX_EXPERTS) return 0;
+  // largest R with moe_dispatch_workspace_bytes(R, E) <= the array: one (E + 1)-word histogram per
+  // wave's chunk of rows
+  const int64_t waves = MOE_STATIC_SCRATCH_BYTES / ((E + 1) * (int64_t)sizeof(int32_t));
+  const int64_t rows = waves * ROWS_PER_WAVE;
+  return rows < ((int64_t)1 << 30) ? rows : ((int64_t)1 << 30);
+}
 
 extern "C" int moe_histogram_scan_static(const int32_t* ids, int64_t R, int64_t E, int32_t* counts,
                                          int32_t* offs, int32_t* pos_to_row, int32_t* row_to_pos,

@@ -876,15 +876,14 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WAVES_PER_SIMD) void grouped_gemm_ker
 using CfgMain = TileCfg<MOE_BM, MOE_BN, MOE_BK, MOE_WM, MOE_WN>;
 
 int compute_units() {
-  static int cus = 0;  // same answer from every thread; a benign race at worst repeats the query
-  if (cus == 0) {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-      n = 256;
-    cus = n;
+  static int cus[MOE_MAX_DEVICES];  // per GPU; 0 = not asked yet
+  const int dev = moe_current_device();
+  if (cus[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cus[dev] = n;
   }
-  return cus;
+  return cus[dev];
 }
 
 // `ntiles` is the number of tile slots; the grid is as many workgroups as are resident at
@@ -894,11 +893,12 @@ int launch(const GemmArgs& a, long long ntiles, hipStream_t s) {
   if (ntiles <= 0) return 0;
   auto kern = grouped_gemm_kernel<MODE, Cfg, OutT>;
   constexpr int LDS = lds_bytes<MODE, Cfg>();
-  static bool attr_done = false;  // idempotent; a benign race at worst repeats the call
-  if (!attr_done) {
+  static bool attr_done[MOE_MAX_DEVICES];  // per GPU and instantiation
+  const int dev = moe_current_device();
+  if (!attr_done[dev]) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
     if (e != hipSuccess) return (int)e;
-    attr_done = true;
+    attr_done[dev] = true;
   }
   // as many workgroups as can be resident at once: the LDS footprint decides how many share a CU
   const long long slots = (long long)compute_units() * ((160 * 1024) / LDS >= Cfg::WGS_PER_CU ? Cfg::WGS_PER_CU : 1);

@@ -382,11 +382,19 @@ extern "C" int moe_rmsnorm_router_fwd(const void* x, int x_dtype, const float* w
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((unsigned)((T + RB - 1) / RB)), block(NT);
   const size_t lds = (size_t)RB * (H + 8) * 2 > (size_t)NW * RB * E * 4 ? (size_t)RB * (H + 8) * 2 : (size_t)NW * RB * E * 4;
+  constexpr int MAX_ROUTER_LDS = RB * (4096 + 8) * 2 > NW * RB * 16 * RMAX_EB * 4 ? RB * (4096 + 8) * 2 : NW * RB * 16 * RMAX_EB * 4;
+  if (lds > (size_t)MAX_ROUTER_LDS) return MOE_ERR_LIMIT;
 #define MOE_NORM_ROUTER(XT, NV)                                                                          \
   do {                                                                                                   \
     auto kern = rmsnorm_router_fwd_kernel<XT, NV>;                                                       \
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
-    if (e != hipSuccess) return (int)e;                                                                  \
+    static bool attr_done[MOE_MAX_DEVICES]; /* per GPU and instantiation: set once, to the largest */    \
+    const int dev = moe_current_device();   /* footprint any supported shape asks for              */    \
+    if (!attr_done[dev]) {                                                                               \
+      hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,  \
+                                         MAX_ROUTER_LDS);                                                \
+      if (e != hipSuccess) return (int)e;                                                                \
+      attr_done[dev] = true;                                                                             \
+    }                                                                                                    \
     hipLaunchKernelGGL(kern, grid, block, lds, s, (const XT*)x, weight, eps, (int)T, (int)(H / 8),       \
                        router_weight, (int)E, (int)k, xn, rstd, logits, ids, gates);                     \
   } while (0)

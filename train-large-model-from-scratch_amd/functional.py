@@ -257,13 +257,18 @@ class _MoEFFN(torch.autograd.Function):
         dyp, _ = ops.combine_bwd(dout, None, gates, pos_to_row, k, row_to_pos)
         dxp, dw1, dw3, dw2, part = _expert_backward(dyp, xp, g, u, act, w1b, w3b, w2b, offs, ctx.w_dtype,
                                                     ctx.needs_input_grad[2:5], ctx.grad_params,
-                                                    ctx.needs_input_grad[1])
+                                                    ctx.needs_input_grad[1] or ctx.needs_input_grad[6])
         dx = ops.permute_bwd(dxp, row_to_pos, T, k, ctx.x_dtype) if ctx.needs_input_grad[0] else None
-        dlogits = None
-        if ctx.needs_input_grad[1]:
+        dlogits = dbias = None
+        if ctx.needs_input_grad[1] or ctx.needs_input_grad[6]:
             dgates = ops.dgates_from_blocks(part, gates, row_to_pos, pos_to_row)
-            dlogits = ops.router_topk_bwd(gates, dgates, ids, T, E, k, ctx.logits_dtype)
-        return dx, dlogits, dw1, dw3, dw2, None, None, None, None
+            if ctx.needs_input_grad[6]:  # column sum of the logits' gradient, before any rounding
+                dl32 = ops.router_topk_bwd(gates, dgates, ids, T, E, k, torch.float32)
+                dbias = dl32.sum(0)
+                dlogits = dl32.to(ctx.logits_dtype) if ctx.needs_input_grad[1] else None
+            else:
+                dlogits = ops.router_topk_bwd(gates, dgates, ids, T, E, k, ctx.logits_dtype)
+        return dx, dlogits, dw1, dw3, dw2, None, dbias, None, None
 
 
 def moe_ffn(x: torch.Tensor, logits: torch.Tensor, w1: torch.Tensor, w3: torch.Tensor,
@@ -272,8 +277,9 @@ def moe_ffn(x: torch.Tensor, logits: torch.Tensor, w1: torch.Tensor, w3: torch.T
     """out[t] = sum_j gate[t,j] * FFN_{e(t,j)}(x[t]).  x [T,H]; logits [T,E]; w1,w3 [E,I,H];
     w2 [E,H,I].  `bias` (fp32 [E]) is added to the logits in fp32 and is part of them from
     there on: both the selection and the softmax over the selected values see logit + bias
-    (a per-expert constant in the router, as benchmark config 2 specifies), and its gradient
-    is the column sum of dlogits.
+    (a per-expert constant in the router, as benchmark config 2 specifies); when it requires a
+    gradient it receives the column sum of the logits' gradient (fp32, summed before that gradient
+    is rounded to the logits' dtype).
     With `return_routing` also returns a dict of the integer routing tensors and gates.
     `bf16_weights`: bf16 copies of (w1, w3, w2) to compute with (None entries are cast here).
     `accumulate_into_grad`: w1, w3, w2 must be leaf tensors; see the module docstring."""
@@ -297,7 +303,8 @@ class _PreNormMoE(torch.autograd.Function):
     (rounded to bf16 once if it is fp32)."""
 
     @staticmethod
-    def forward(ctx, x, norm_w, wr, w1, w3, w2, eps, k, bias, shadows, grad_params, add_residual):
+    def forward(ctx, x, norm_w, wr, w1, w3, w2, eps, k, bias, shadows, grad_params, add_residual,
+                fused_router):
         T, H = x.shape
         E = wr.shape[0]
         x = _dense(x)
@@ -305,11 +312,12 @@ class _PreNormMoE(torch.autograd.Function):
         w1b, w3b, w2b = (sh if sh is not None else ops.cast_bf16(_dense(w))
                          for w, sh in zip((w1, w3, w2), shadows))
         wrb = wr.detach().to(torch.bfloat16)
-        if norm_w is not None and bias is None and T > 0 and ops.rmsnorm_router_supported(H, E, k):
+        if (fused_router and norm_w is not None and bias is None and T > 0
+                and ops.rmsnorm_router_supported(H, E, k)):
             # norm, router product and selection in one kernel: the normalised rows are not read
             # a second time for the router, the logits are selected on before they leave the chip
             nw = norm_w.detach().float().contiguous()
-            xn, rstd, logits, ids, gates = ops.rmsnorm_router_fwd(x, nw, eps, wrb.contiguous(), k)
+            xn, rstd, logits, ids, gates = ops.rmsnorm_router_fwd(x, nw, eps, _dense(wrb), k)
         else:
             if norm_w is not None:
                 nw = norm_w.detach().float().contiguous()
@@ -357,9 +365,19 @@ class _PreNormMoE(torch.autograd.Function):
         dxp, dw1, dw3, dw2, part = _expert_backward(dyp, xp, g, u, act, w1b, w3b, w2b, offs, ctx.w_dtype,
                                                     ctx.needs_input_grad[3:6], ctx.grad_params, True)
         dgates = ops.dgates_from_blocks(part, gates, row_to_pos, pos_to_row)
-        dlogits = ops.router_topk_bwd(gates, dgates, ids, T, E, k, torch.bfloat16)
-        if dlogits_ext is not None:
-            dlogits = dlogits + dlogits_ext.to(dlogits.dtype)
+        dbias = None
+        if ctx.needs_input_grad[8]:
+            # the bias is a per-expert constant added to the logits (in fp32): its gradient is the
+            # column sum of the logits' gradient, taken before that is rounded to bf16
+            dl32 = ops.router_topk_bwd(gates, dgates, ids, T, E, k, torch.float32)
+            if dlogits_ext is not None:
+                dl32 = dl32 + dlogits_ext.float()
+            dbias = dl32.sum(0)
+            dlogits = dl32.to(torch.bfloat16)
+        else:
+            dlogits = ops.router_topk_bwd(gates, dgates, ids, T, E, k, torch.bfloat16)
+            if dlogits_ext is not None:
+                dlogits = dlogits + dlogits_ext.to(dlogits.dtype)
         dwr = _router_wgrad(dlogits, xn, ctx.wr_dtype) if ctx.needs_input_grad[2] else None
         dx = dnw = None
         if ctx.needs_input_grad[0] or (ctx.has_norm and ctx.needs_input_grad[1]):
@@ -375,22 +393,25 @@ class _PreNormMoE(torch.autograd.Function):
                     dx = dx + dout
             if not ctx.needs_input_grad[0]:
                 dx = None
-        return dx, dnw, dwr, dw1, dw3, dw2, None, None, None, None, None, None
+        return dx, dnw, dwr, dw1, dw3, dw2, None, None, dbias, None, None, None, None
 
 
 def prenorm_moe(x: torch.Tensor, norm_weight: torch.Tensor, router_weight: torch.Tensor,
                 w1: torch.Tensor, w3: torch.Tensor, w2: torch.Tensor, k: int, eps: float = 1e-6,
                 add_residual: bool = True, bf16_weights=None, accumulate_into_grad: bool = False,
-                return_routing: bool = False):
+                return_routing: bool = False, fused_router: bool = True):
     """(x + MoE(RMSNorm(x)), router logits) for x [T,H]: model/gpt.py:32-33 with
     model/modules/norm.py:14-19 and model/modules/mlp.py:95-169 in one differentiable call.
     Router logits are bf16 (what the reference produces under its bf16 autocast); the output
-    has the dtype of x.  H <= 8192."""
+    has the dtype of x.  H <= 8192.  `fused_router=False` takes the logits from the library's
+    product (bit-identical to what `routed_moe` and `MoE.forward` select on) instead of the fused
+    norm+router kernel, whose own summation order can move a bf16 logit by one unit in the last
+    place."""
     grad_params = None
     if accumulate_into_grad:
         grad_params = tuple(w if (w.requires_grad and w.is_leaf) else None for w in (w1, w3, w2))
     res = _PreNormMoE.apply(x, norm_weight, router_weight, w1, w3, w2, float(eps), k, None, bf16_weights,
-                            grad_params, add_residual)
+                            grad_params, add_residual, fused_router)
     if return_routing:
         return res[0], res[1], dict(zip(_ROUTING_NAMES, res[2:]))
     return res[0], res[1]
@@ -409,7 +430,7 @@ def routed_moe(x: torch.Tensor, router_weight: torch.Tensor, w1: torch.Tensor, w
     if accumulate_into_grad:
         grad_params = tuple(w if (w.requires_grad and w.is_leaf) else None for w in (w1, w3, w2))
     res = _PreNormMoE.apply(x, None, router_weight, w1, w3, w2, 0.0, k, bias, bf16_weights, grad_params,
-                            False)
+                            False, True)
     if return_routing:
         return res[0], res[1], dict(zip(_ROUTING_NAMES, res[2:]))
     return res[0], res[1]

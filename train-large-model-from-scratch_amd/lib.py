@@ -18,6 +18,7 @@ SIGNATURES = {
     "moe_histogram_scan": (_int, [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _vp]),
     "moe_histogram_scan_checked": (_int, [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp]),
     "moe_static_scratch_bytes": (_i64, []),
+    "moe_static_scratch_max_rows": (_i64, [_i64]),
     "moe_histogram_scan_static": (_int, [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp]),
     "moe_permute_fwd": (_int, [_vp, _int, _vp, _i64, _i64, _i64, _vp, _vp]),
     "moe_permute_fwd_scatter": (_int, [_vp, _int, _vp, _i64, _i64, _i64, _vp, _vp]),

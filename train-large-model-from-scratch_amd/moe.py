@@ -72,6 +72,10 @@ class MoE(nn.Module):
         # instead of by autograd (saves a pass over them per gradient-accumulation micro-step;
         # hooks on these three parameters then do not run, see functional.py).
         self.accumulate_wgrad_into_grad = False
+        # False: `forward_prenorm` takes the router logits from the library's product (the one
+        # `forward` uses) instead of the fused norm+router kernel, whose summation order can move
+        # a bf16 logit by one unit in the last place and with it the routing of a near-tie.
+        self.fused_router = True
         self._init_expert_weights(config.seed)
 
     def _init_expert_weights(self, base_seed: int):
@@ -150,6 +154,10 @@ class MoE(nn.Module):
                           self.experts_down_weights, self.top_k, bf16_weights=self._bf16_operands(),
                           accumulate_into_grad=self.accumulate_wgrad_into_grad)
 
+    def _router_has_hooks(self) -> bool:
+        r = self.router
+        return bool(r._forward_hooks or r._forward_pre_hooks or r._backward_hooks or r._backward_pre_hooks)
+
     def _router_in_bf16(self, x: torch.Tensor) -> bool:
         """Whether `self.router(x)` would be a bf16 product anyway (bf16 autocast, or bf16
         tensors): then router and experts run as one autograd node."""
@@ -168,6 +176,12 @@ class MoE(nn.Module):
                                  self.experts_gate_weights, self.experts_up_weights,
                                  self.experts_down_weights, self.top_k)
             return out.reshape(B, T, D), gate_logits
+        if self._router_has_hooks():
+            # hooks on the nn.Linear fire only if it is called: the product is the module's own
+            # (mlp.py:100), the logits go to the expert function as in the reference
+            gate_logits = self.router(x)
+            out = self._experts(x.reshape(B * T, D), gate_logits.reshape(B * T, self.num_experts))
+            return out.reshape(B, T, D), gate_logits
         if self._router_in_bf16(x):
             out, gate_logits = self._layer(x.reshape(B * T, D))
             return out.reshape(B, T, D), gate_logits.reshape(B, T, self.num_experts)
@@ -185,12 +199,15 @@ class MoE(nn.Module):
         calling the three pieces separately under bf16 autocast; the residual stream is read
         once on the way in and written once on the way out."""
         B, T, D = x.size()
-        if D > 8192:  # wider than the fused norm kernels hold in registers: the separate calls
+        if D > 8192 or self._router_has_hooks():
+            # wider than the fused norm kernels hold in registers, or hooks on the router that only
+            # a call of the nn.Linear runs: the separate calls
             out, logits = self(norm(x))
             return (x + out if add_residual else out), logits
         out, logits = prenorm_moe(x.reshape(B * T, D), norm.weight, self.router.weight,
                                   self.experts_gate_weights, self.experts_up_weights,
                                   self.experts_down_weights, self.top_k, eps=norm.variance_epsilon,
                                   add_residual=add_residual, bf16_weights=self._bf16_operands(),
-                                  accumulate_into_grad=self.accumulate_wgrad_into_grad)
+                                  accumulate_into_grad=self.accumulate_wgrad_into_grad,
+                                  fused_router=self.fused_router)
         return out.reshape(B, T, D), logits.reshape(B, T, self.num_experts)
