@@ -38,6 +38,8 @@ MEASURED_HBM_BYTES_PER_LAUNCH = {
     (3, "gemm_dgrad_down_swiglu_bwd_packed"): 2.465e9,
     (3, "gemm_dgrad_gateup_packed"): 3.771e9,
     (3, "gemm_wgrad_pair"): 2.23e9,
+    (3, "gemm_gateup_swiglu_fwd_blocked"): 4.009e9,
+    (3, "gemm_dgrad_down_swiglu_bwd_blocked"): 2.465e9,
 }
 
 
@@ -100,7 +102,7 @@ def _moe_dominant_kernel(torch, P, s, x_bf16, wr_bf16, ws_bf16):
         ids, _ = ops.router_topk(logits, s.k, None)
         _, offs, p2r, r2p = ops.histogram_scan(ids, s.E)
         xp = ops.permute_fwd(x_bf16, p2r, s.k, r2p)
-        ms = _event_time_ms(torch, lambda: ops.gemm_gateup(xp, ws_bf16[0], ws_bf16[1], offs, True), 10, 2)
+        ms = _event_time_ms(torch, lambda: ops.gemm_gateup_blocked(xp, ws_bf16[0], ws_bf16[1], offs), 10, 2)
     fl = 4 * s.R * s.H * s.I
     return {"kernel": "gemm_gateup_swiglu_fwd", "bound": "mfma", "achieved": round(fl / ms / 1e9, 1),
             "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(fl / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
@@ -467,7 +469,7 @@ def main():
                 _, offs, p2r, r2p = ops.histogram_scan(rids, s.E)
                 kk = s.k
             xp = ops.permute_fwd(xd, p2r, kk, r2p)
-            g, u, act = ops.gemm_gateup(xp, w1, w3, offs, True)
+            gu, act = ops.gemm_gateup_blocked(xp, w1, w3, offs)
             y = ops.gemm_down(act, w2, offs)
             dyy = dy if dy is not None else torch.randn_like(xd)
             dyp, _ = ops.combine_bwd(dyy, None, gates, p2r, kk, r2p)
@@ -476,22 +478,22 @@ def main():
             # their two weight gradients are then one launch)
             packed = s.I % 256 == 0
             if packed:
-                dgu = ops.gemm_dgrad_down_packed(dyp, w2, g, u, offs, dgate_blocks=routed)[0]
+                dgu = ops.gemm_dgrad_down_blocked(dyp, w2, gu, offs, dgate_blocks=routed, packed=True)[0]
                 dxp = ops.gemm_dgrad_gateup_packed(dgu, w1, w3, offs)
                 dg = dgu[:, :s.I].contiguous()
             else:
-                dg, du = ops.gemm_dgrad_down(dyp, w2, g, u, offs, dgate_blocks=routed)[:2]
+                dg, du = ops.gemm_dgrad_down_blocked(dyp, w2, gu, offs, dgate_blocks=routed)[:2]
                 dxp = ops.gemm_dgrad_gateup(dg, du, w1, w3, offs)
             bf = torch.bfloat16
             a = 2  # bytes per bf16 element
             T, R, H, I, E = xd.shape[0], s.R, s.H, s.I, s.E
             kernels = [
                 # name, callable, algorithmic flops, algorithmic bytes, launches per step
-                ("gemm_gateup_swiglu_fwd", lambda: ops.gemm_gateup(xp, w1, w3, offs, True), 4 * RHI, 0, 1),
+                ("gemm_gateup_swiglu_fwd", lambda: ops.gemm_gateup_blocked(xp, w1, w3, offs), 4 * RHI, 0, 1),
                 ("gemm_down_fwd", lambda: ops.gemm_down(act, w2, offs), 2 * RHI, 0, 1),
                 ("gemm_dgrad_down_swiglu_bwd",
-                 (lambda: ops.gemm_dgrad_down_packed(dyp, w2, g, u, offs, dgate_blocks=routed)) if packed else
-                 (lambda: ops.gemm_dgrad_down(dyp, w2, g, u, offs, dgate_blocks=routed)), 2 * RHI, 0, 1),
+                 (lambda: ops.gemm_dgrad_down_blocked(dyp, w2, gu, offs, dgate_blocks=routed, packed=packed)),
+                 2 * RHI, 0, 1),
                 ("gemm_dgrad_gateup",
                  (lambda: ops.gemm_dgrad_gateup_packed(dgu, w1, w3, offs)) if packed else
                  (lambda: ops.gemm_dgrad_gateup(dg, du, w1, w3, offs)), 4 * RHI, 0, 1),
@@ -554,7 +556,9 @@ def main():
     # loops above stay beside them
     in_step_recs = []
     if in_step:
-        gemm_flops_of = {"moe_gemm_gateup_swiglu_fwd": 4, "moe_gemm_down_fwd": 2, "moe_gemm_dgrad_down_swiglu_bwd": 2,
+        gemm_flops_of = {"moe_gemm_gateup_swiglu_fwd": 4, "moe_gemm_gateup_swiglu_fwd_blocked": 4,
+                         "moe_gemm_dgrad_down_swiglu_bwd_blocked": 2,
+                         "moe_gemm_down_fwd": 2, "moe_gemm_dgrad_down_swiglu_bwd": 2,
                          "moe_gemm_dgrad_down_swiglu_bwd_dgate": 2, "moe_gemm_dgrad_down_swiglu_bwd_packed": 2,
                          "moe_gemm_dgrad_gateup": 4, "moe_gemm_dgrad_gateup_packed": 4, "moe_gemm_wgrad_pair": 4,
                          "moe_gemm_wgrad": 2}

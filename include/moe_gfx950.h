@@ -171,6 +171,27 @@ int moe_dgates_from_blocks(const float* dgate_part, int64_t blocks, const float*
  * blocks are read coalesced and only the 4-byte results are scattered (mlp.py:166 backward). */
 int moe_dgates_from_blocks_by_pos(const float* dgate_part, int64_t blocks, const float* gates,
                                   const int32_t* pos_to_row, int64_t R, float* dgates, void* stream);
+/* g and u in a layout private to the library.  Nothing but the SwiGLU backward reads the two
+ * pre-activation planes the forward saves (mlp.py:154-156 under autograd keeps them as [R, I]
+ * tensors), so they need not be rows: gu_blocked holds one 4 KB record per 32 x 32 block of every
+ * 256-row tile of the expert-contiguous rows, g and u of the block together, each in the order in
+ * which a wavefront's matrix-core accumulators hold it.  The forward kernel stores the records
+ * straight from its registers and the backward kernel loads them straight into the layout it
+ * computes in; act, dg, du and dgate_part are the same bits as from the row-major entry points.
+ * The buffer is opaque to the caller: moe_gu_blocked_bytes(R, E, I) bytes (it depends on R, E and
+ * I only, never on the routing: (ceil(R/256) + E) * 256 rows are provided for), 16-byte aligned,
+ * written by moe_gemm_gateup_swiglu_fwd_blocked and valid for moe_gemm_dgrad_down_swiglu_bwd_blocked
+ * with the same offs, E, R and I.  dg and du [R, ld_out] rows (ld_out = 0 means I; 2*I with
+ * du = dg + I gives the side-by-side buffer of moe_gemm_wgrad_pair); dgate_part may be NULL. */
+int64_t moe_gu_blocked_bytes(int64_t R, int64_t E, int64_t I);
+int moe_gemm_gateup_swiglu_fwd_blocked(const uint16_t* xp, const uint16_t* w1, const uint16_t* w3,
+                                       const int32_t* offs, int64_t E, int64_t R, int64_t H,
+                                       int64_t I, void* gu_blocked, uint16_t* act, void* stream);
+int moe_gemm_dgrad_down_swiglu_bwd_blocked(const uint16_t* dyp, const uint16_t* w2,
+                                           const void* gu_blocked, const int32_t* offs, int64_t E,
+                                           int64_t R, int64_t H, int64_t I, uint16_t* dg,
+                                           uint16_t* du, int64_t ld_out, float* dgate_part,
+                                           void* stream);
 /* Backward of gate/up w.r.t. the rows (autograd of mlp.py:154-155): dxp = dg*W1 + du*W3. */
 int moe_gemm_dgrad_gateup(const uint16_t* dg, const uint16_t* du, const uint16_t* w1,
                           const uint16_t* w3, const int32_t* offs, int64_t E, int64_t R,

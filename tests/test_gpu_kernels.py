@@ -388,6 +388,21 @@ def test_expert_gemms_forward_backward(ops, R, H, I, E, empty):
         ref_du[a:b] = dact * gf[a:b] * s
         ref_dw2[e] = dyp[a:b].float().t() @ af[a:b]
     assert _close(dg, ref_dg) and _close(du, ref_du)
+    # g and u in the library's blocked layout (what the autograd functions save): the forward's
+    # act and every result of the backward kernel must be the same bits as with [R, I] rows,
+    # separate or side by side, with and without the gate gradients' block sums
+    gu, act_b = ops.gemm_gateup_blocked(xp.cuda(), w1.cuda(), w3.cuda(), offs)
+    assert torch.equal(act_b, act)
+    dg_r, du_r, part_r = ops.gemm_dgrad_down(dyp.cuda(), w2.cuda(), g, u, offs, dgate_blocks=True)
+    assert torch.equal(dg_r, dg) and torch.equal(du_r, du)
+    dg_b, du_b, part_b = ops.gemm_dgrad_down_blocked(dyp.cuda(), w2.cuda(), gu, offs, dgate_blocks=True)
+    assert torch.equal(dg_b, dg) and torch.equal(du_b, du)
+    assert torch.equal(part_b.view(torch.int32), part_r.view(torch.int32))
+    dg_b2, du_b2, none = ops.gemm_dgrad_down_blocked(dyp.cuda(), w2.cuda(), gu, offs)
+    assert none is None and torch.equal(dg_b2, dg) and torch.equal(du_b2, du)
+    dgu_b, part_b3 = ops.gemm_dgrad_down_blocked(dyp.cuda(), w2.cuda(), gu, offs, dgate_blocks=True, packed=True)
+    assert torch.equal(dgu_b[:, :I], dg) and torch.equal(dgu_b[:, I:], du)
+    assert torch.equal(part_b3.view(torch.int32), part_r.view(torch.int32))
     dxp = ops.gemm_dgrad_gateup(dg, du, w1.cuda(), w3.cuda(), offs)
     dgf, duf = dg.float().cpu(), du.float().cpu()
     ref_dxp = torch.zeros(R, H)

@@ -163,6 +163,7 @@ _OPTIONAL_POINTERS = {
     "moe_histogram_scan_checked": {"bad_ids"}, "moe_histogram_scan_static": {"bad_ids"},
     "moe_permute_bwd": {"addend"},
     "moe_gemm_dgrad_down_swiglu_bwd_packed": {"dgate_part"},
+    "moe_gemm_dgrad_down_swiglu_bwd_blocked": {"dgate_part"},
     "moe_combine_fwd": {"gates"}, "moe_combine_fwd_residual": {"gates"},
     "moe_combine_bwd": {"gates"}, "moe_combine_bwd_by_token": {"gates"},
     "moe_rmsnorm_bwd": {"d2", "dres"},

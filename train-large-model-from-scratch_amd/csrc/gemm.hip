@@ -204,8 +204,15 @@ constexpr int lds_bytes() {
 
 constexpr int GEMM_MAX_E = 1024;  // per-expert tile prefix lives in LDS
 
-template <int MODE, typename Cfg, typename OutT>
+// BLK (GATEUP and DGRAD_DOWN only): g and u, which nothing but the SwiGLU backward reads, are kept
+// in a layout private to the library instead of as [R, I] rows: one 4 KB record per 32 x 32 block
+// of a row tile, holding the block exactly as the matrix cores leave it in a wave's accumulators
+// (see gu_block below).  The forward kernel then stores them straight from its registers and the
+// backward kernel loads them straight into the layout it computes in: neither passes them
+// through LDS.
+template <int MODE, typename Cfg, typename OutT, bool BLK = false>
 __global__ __launch_bounds__(Cfg::NT, Cfg::WAVES_PER_SIMD) void grouped_gemm_kernel(const GemmArgs p) {
+  static_assert(!BLK || MODE == GATEUP || MODE == DGRAD_DOWN, "only g and u have the blocked layout");
   constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, NT = Cfg::NT, KS = Cfg::KS;
   constexpr int FM = Cfg::FM, FN = Cfg::FN, WTM = Cfg::WTM, WTN = Cfg::WTN;
   constexpr bool DUAL = (MODE == GATEUP);
@@ -226,9 +233,10 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WAVES_PER_SIMD) void grouped_gemm_ker
   uint16_t* sA = smem;                       // [2][StA::LDS_ELEMS]
   uint16_t* sB = smem + 2 * StA::LDS_ELEMS;  // [2][StB::LDS_ELEMS]
 
-  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  // (the wave's index is the same in all of its lanes: read it once so that everything derived
+  // from it lives in scalar registers)
+  const int lane = threadIdx.x & 63, wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const int wm = wv / Cfg::WN, wn = wv % Cfg::WN;
-  const int l32 = lane & 31, lh = lane >> 5;
 
   // ---- which tiles this workgroup computes
   // The kernel is persistent: the grid has one workgroup per compute unit and each walks a
@@ -330,7 +338,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WAVES_PER_SIMD) void grouped_gemm_ker
   }
 
   struct Tile {
-    int e, row0, row_end, n0, m0;
+    int e, row0, row_end, n0, m0, slot;
     int Kseg, kt_per_seg, nkt;
     bool need_mask;
     View vA0, vA1, vB0, vB1;
@@ -346,6 +354,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WAVES_PER_SIMD) void grouped_gemm_ker
     const int n_tile = logical % p.n_tiles;
     const int slot = logical / p.n_tiles;
     t.m0 = 0;
+    t.slot = slot;
     if constexpr (MODE == WGRAD) {
       t.e = slot / p.m_slots;
       t.m0 = (slot % p.m_slots) * BM;
@@ -568,7 +577,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WAVES_PER_SIMD) void grouped_gemm_ker
   constexpr int OSZ = (MODE == WGRAD) ? (int)sizeof(OutT) : 2;
   constexpr int SSTRIDE = WTNC * OSZ + 16;  // bytes per strip row (16 bytes of padding)
   constexpr int SBYTES = 32 * SSTRIDE;
-  constexpr int NSTRIP = (MODE == GATEUP) ? 3 : (MODE == DGRAD_DOWN ? 2 : 1);
+  constexpr int NSTRIP = (MODE == GATEUP) ? (BLK ? 1 : 3) : (MODE == DGRAD_DOWN ? 2 : 1);
   constexpr int CPRO = WTNC * OSZ / 16;  // 16-byte chunks per strip row
   constexpr int RPI = 64 / CPRO;         // rows covered by one wave-wide 16-byte access
   static_assert(64 % CPRO == 0 && 32 % RPI == 0, "strip shape");
@@ -590,13 +599,6 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WAVES_PER_SIMD) void grouped_gemm_ker
                     : reinterpret_cast<char*>(smem) + wv * (NSTRIP * SBYTES);
   const int ldc = p.ld_c ? p.ld_c : p.N;  // outputs
   const int ldx = p.N;                    // epilogue inputs (g, u)
-  auto acc_ptr = [&](int plane, int j, int q) {  // 4 consecutive columns in accumulator layout
-    return strip + plane * SBYTES + l32 * SSTRIDE + (j * 32 + 8 * q + 4 * lh) * OSZ;
-  };
-  auto put4 = [&](int plane, int j, int q, float a, float b, float c, float d) {
-    if constexpr (OSZ == 4) *reinterpret_cast<f32x4*>(acc_ptr(plane, j, q)) = f32x4{a, b, c, d};
-    else *reinterpret_cast<u32x2*>(acc_ptr(plane, j, q)) = u32x2{pack_bf16x2(a, b), pack_bf16x2(c, d)};
-  };
   // The accumulators of a strip are cleared for the next tile as soon as they are in LDS: the
   // moves fill the waits of the strip's LDS and global traffic instead of a slot before the
   // next main loop.
@@ -606,9 +608,36 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WAVES_PER_SIMD) void grouped_gemm_ker
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
   };
+  // Blocked g/u (BLK): record of the 32 x 32 block (row block rb of row-tile slot `slot`, column
+  // block cb = column / 32), GU_BLOCK_BYTES each: [g: q0q1 of lanes 0..63 | g: q2q3 | u: q0q1 |
+  // u: q2q3], 16 bytes per lane and part, where lane l of the wave that owns the block holds row
+  // l % 32 and columns 8*q + 4*(l/32) .. +3 of it for q = 0..3 (the accumulator layout above).
+  // A wave-wide 16-byte access to one part covers 1 KB of consecutive addresses.  Row tiles are
+  // numbered as the tile list numbers them (expert by expert, BM rows each), so that the forward
+  // and the backward kernel agree on `slot` from the offsets alone.
+  constexpr int GU_BLOCK_BYTES = 4096;
+  const int n_cb = (p.N + 31) / 32;
+  auto gu_block = [&](const void* base, const Tile& t, int rb, int cb, int ln) {
+    return (char*)base + (((long long)t.slot * (BM / 32) + rb) * n_cb + cb) * GU_BLOCK_BYTES + ln * 16;
+  };
   // `halfway` runs once, after the second of the FM strips; `last_rows_in` once the SwiGLU-backward
   // epilogue has taken the last g/u rows out of their registers
   auto epilogue = [&](const Tile& t, auto&& halfway, auto&& last_rows_in) {
+    // Every per-lane address of the epilogue is derived from this copy of the lane index, which
+    // the empty asm makes opaque: the compiler then recomputes them here, a handful of integer
+    // operations per tile, instead of hoisting them out of the tile loop and holding a dozen
+    // registers through the main loop for them.
+    int lane_e = lane;
+    asm volatile("" : "+v"(lane_e));
+    const int l32 = lane_e & 31, lh = lane_e >> 5;
+    const int row_in_pass = lane_e / CPRO, chunk_in_row = lane_e % CPRO;
+    auto acc_ptr = [&](int plane, int j, int q) {  // 4 consecutive columns in accumulator layout
+      return strip + plane * SBYTES + l32 * SSTRIDE + (j * 32 + 8 * q + 4 * lh) * OSZ;
+    };
+    auto put4 = [&](int plane, int j, int q, float a, float b, float c, float d) {
+      if constexpr (OSZ == 4) *reinterpret_cast<f32x4*>(acc_ptr(plane, j, q)) = f32x4{a, b, c, d};
+      else *reinterpret_cast<u32x2*>(acc_ptr(plane, j, q)) = u32x2{pack_bf16x2(a, b), pack_bf16x2(c, d)};
+    };
     const int col_w0 = t.n0 + wn * WTNC;  // first output column of the wave
     char* C0 = (char*)p.C0;
     int m_shift = 0;  // WGRAD with two results: the rows of the second one start at m_split
@@ -632,7 +661,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WAVES_PER_SIMD) void grouped_gemm_ker
       const int rbase = (MODE == WGRAD ? t.m0 : t.row0) + wm * WTM + i * 32;
 #pragma unroll
       for (int it = 0; it < 32 / RPI; ++it) {
-        const int rr = it * RPI + lane / CPRO, ch = lane % CPRO;
+        const int rr = it * RPI + row_in_pass, ch = chunk_in_row;
         const u32x4 v = *reinterpret_cast<const u32x4*>(strip + plane * SBYTES + rr * SSTRIDE + ch * 16);
         const int r = rbase + rr, c = col_w0 + ch * (16 / OSZ);
         if (r < row_lim && c < p.N) {
@@ -664,7 +693,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WAVES_PER_SIMD) void grouped_gemm_ker
       const int rbase = t.row0 + wm * WTM + i * 32;
 #pragma unroll
       for (int it = 0; it < 32 / RPI; ++it) {
-        const int rr = it * RPI + lane / CPRO, ch = lane % CPRO;
+        const int rr = it * RPI + row_in_pass, ch = chunk_in_row;
         const int r = rbase + rr, c = col_w0 + ch * (16 / OSZ);
         rr_.g[it] = u32x4{0, 0, 0, 0};
         rr_.u[it] = u32x4{0, 0, 0, 0};
@@ -677,18 +706,43 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WAVES_PER_SIMD) void grouped_gemm_ker
     auto rows_to_strip = [&](const RowRegs& rr_) {
 #pragma unroll
       for (int it = 0; it < 32 / RPI; ++it) {
-        const int rr = it * RPI + lane / CPRO, ch = lane % CPRO;
+        const int rr = it * RPI + row_in_pass, ch = chunk_in_row;
         *reinterpret_cast<u32x4*>(strip + 0 * SBYTES + rr * SSTRIDE + ch * 16) = rr_.g[it];
         *reinterpret_cast<u32x4*>(strip + 1 * SBYTES + rr * SSTRIDE + ch * 16) = rr_.u[it];
       }
     };
+    // (BLK) the two 16-byte parts of g and of u for each of the strip's column blocks
+    struct BlkRegs {
+      u32x4 g[FNC][2], u[FNC][2];
+    };
+    auto request_block = [&](int i, int j, BlkRegs& b) {
+      const int cb = (col_w0 + j * 32) / 32;
+      const u32x4 zero = u32x4{0, 0, 0, 0};
+      b.g[j][0] = b.g[j][1] = b.u[j][0] = b.u[j][1] = zero;
+      if (t.row0 + wm * WTM + i * 32 < t.row_end && cb < n_cb) {
+        const u32x4* rec = reinterpret_cast<const u32x4*>(gu_block(p.X0, t, wm * FM + i, cb, lane_e));
+        b.g[j][0] = rec[0];
+        b.g[j][1] = rec[64];
+        b.u[j][0] = rec[128];
+        b.u[j][1] = rec[192];
+      }
+    };
     RowRegs rows_in;
-    if constexpr (MODE == DGRAD_DOWN) request_rows(0, rows_in);
+    BlkRegs blk_in;
+    if constexpr (MODE == DGRAD_DOWN && BLK) {
+#pragma unroll
+      for (int j = 0; j < FNC; ++j) request_block(0, j, blk_in);
+    } else if constexpr (MODE == DGRAD_DOWN) {
+      request_rows(0, rows_in);
+    }
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
       if constexpr (MODE == GATEUP) {
+        // (BLK) blocks of a strip that starts past the end of the expert's rows are never read
+        const bool strip_live = t.row0 + wm * WTM + i * 32 < t.row_end;
 #pragma unroll
-        for (int j = 0; j < FNC; ++j)
+        for (int j = 0; j < FNC; ++j) {
+          u32x2 gq[2], uq[2];
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
             float g[4], u[4], a[4];
@@ -699,17 +753,71 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WAVES_PER_SIMD) void grouped_gemm_ker
               a[x] = g[x] * sigmoidf_(g[x]) * u[x];
             }
             put4(0, j, q, a[0], a[1], a[2], a[3]);
-            if (p.C0) {
+            if constexpr (BLK) {
+              gq[q & 1] = u32x2{pack_bf16x2(g[0], g[1]), pack_bf16x2(g[2], g[3])};
+              uq[q & 1] = u32x2{pack_bf16x2(u[0], u[1]), pack_bf16x2(u[2], u[3])};
+              if (q & 1) {  // a 16-byte part of the record is complete: it leaves at once
+                const int cb = (col_w0 + j * 32) / 32;
+                if (p.C0 && strip_live && cb < n_cb) {
+                  u32x4* rec = reinterpret_cast<u32x4*>(gu_block(p.C0, t, wm * FM + i, cb, lane_e));
+                  rec[64 * (q >> 1)] = u32x4{gq[0][0], gq[0][1], gq[1][0], gq[1][1]};
+                  rec[128 + 64 * (q >> 1)] = u32x4{uq[0][0], uq[0][1], uq[1][0], uq[1][1]};
+                }
+              }
+            } else if (p.C0) {
               put4(1, j, q, g[0], g[1], g[2], g[3]);
               put4(2, j, q, u[0], u[1], u[2], u[3]);
             }
           }
+        }
         zero_row(i);
         store_rows(0, i, (char*)p.C2);
-        if (p.C0) {
-          store_rows(1, i, (char*)p.C0);
-          store_rows(2, i, (char*)p.C1);
+        if constexpr (!BLK) {
+          if (p.C0) {
+            store_rows(1, i, (char*)p.C0);
+            store_rows(2, i, (char*)p.C1);
+          }
         }
+      } else if constexpr (MODE == DGRAD_DOWN && BLK) {
+        // g and u arrive in the accumulator layout: nothing to rearrange.  The registers of column
+        // block j are asked for the next strip's block as soon as this strip's block is computed.
+        float rowdot = 0.f;
+#pragma unroll
+        for (int j = 0; j < FNC; ++j) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const u32x4 gv = blk_in.g[j][q >> 1], uv = blk_in.u[j][q >> 1];
+            const uint32_t g01 = gv[2 * (q & 1)], g23 = gv[2 * (q & 1) + 1];
+            const uint32_t u01 = uv[2 * (q & 1)], u23 = uv[2 * (q & 1) + 1];
+            const float g[4] = {bf16lo(g01), bf16hi(g01), bf16lo(g23), bf16hi(g23)};
+            const float u[4] = {bf16lo(u01), bf16hi(u01), bf16lo(u23), bf16hi(u23)};
+            float dg[4], du[4];
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+              const float dact = acc[i][j][4 * q + x];
+              const float sg = sigmoidf_(g[x]);
+              const float gs = g[x] * sg;                     // silu(g)
+              du[x] = dact * gs;
+              dg[x] = (dact * u[x]) * (sg + (gs - gs * sg));  // silu'(g) = s + g*s*(1-s)
+              rowdot += du[x] * u[x];                         // dact * act
+            }
+            put4(0, j, q, dg[0], dg[1], dg[2], dg[3]);
+            put4(1, j, q, du[0], du[1], du[2], du[3]);
+          }
+          __builtin_amdgcn_sched_barrier(0);  // (the loads must not move up: their registers are in use)
+          if (i + 1 < FM) request_block(i + 1, j, blk_in);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        if (i + 1 == FM) last_rows_in();
+        {
+          rowdot += __shfl_xor(rowdot, 32, MOE_WAVE);
+          const int r = t.row0 + wm * WTM + i * 32 + l32;
+          if (lh == 0 && r < row_lim && p.C2)
+            reinterpret_cast<float*>(p.C2)[(long long)((t.n0 / BNC) * Cfg::WN + wn) * p.R + r] = rowdot;
+        }
+        zero_row(i);
+        store_rows(0, i, (char*)p.C0);
+        store_rows(1, i, (char*)p.C1);
       } else if constexpr (MODE == DGRAD_DOWN) {
         rows_to_strip(rows_in);
         if (i + 1 < FM) request_rows(i + 1, rows_in);
@@ -767,7 +875,14 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WAVES_PER_SIMD) void grouped_gemm_ker
   // At the top of the loop the first k-tile of `cur` is already on its way into the staging
   // registers (requested before the previous tile's epilogue).
   auto request_first = [&](const Tile& t) {
-    if (0 < t.nkt) load_tile(t, 0, stg);
+    if (0 < t.nkt) {
+      load_tile(t, 0, stg);
+    } else {
+      // (nothing will be read from the staging registers: say so, or they stay alive through the
+      // epilogue on account of this path)
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) asm volatile("" : "=v"(stg.v[c]));
+    }
   };
   Tile cur;
   if (t_next >= t_hi || !locate(t_next, cur)) return;
@@ -780,6 +895,17 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WAVES_PER_SIMD) void grouped_gemm_ker
     // multiplies nothing: it only keeps moving operand chunks and meets the barriers (the
     // same ones in the same order as the waves that work), so that such a tile costs the
     // matrix pipe half of a full one.
+    // The fragment registers carry nothing from one tile to the next.  The compiler cannot see that
+    // (their first reads sit behind conditions it does not correlate with the loops that use them)
+    // and would keep all of them alive through the epilogue; an empty asm that "writes" them ends
+    // their live ranges here at no cost.
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+#pragma unroll
+      for (int i = 0; i < FM; ++i) asm volatile("" : "=v"(fr[h].a[i]));
+#pragma unroll
+      for (int j = 0; j < FN; ++j) asm volatile("" : "=v"(fr[h].b[j]));
+    }
     const bool idle =
         (MODE != WGRAD) && __builtin_amdgcn_readfirstlane((int)(wm * WTM >= cur.row_end - cur.row0)) != 0;
     // where the next tile lies is worked out now (a binary search in LDS and some address
@@ -888,10 +1014,10 @@ int compute_units() {
 
 // `ntiles` is the number of tile slots; the grid is as many workgroups as are resident at
 // once (one or two per compute unit, by LDS footprint), or fewer when there are fewer tiles.
-template <int MODE, typename Cfg, typename OutT>
+template <int MODE, typename Cfg, typename OutT, bool BLK = false>
 int launch(const GemmArgs& a, long long ntiles, hipStream_t s) {
   if (ntiles <= 0) return 0;
-  auto kern = grouped_gemm_kernel<MODE, Cfg, OutT>;
+  auto kern = grouped_gemm_kernel<MODE, Cfg, OutT, BLK>;
   constexpr int LDS = lds_bytes<MODE, Cfg>();
   static bool attr_done[MOE_MAX_DEVICES];  // per GPU and instantiation
   const int dev = moe_current_device();
@@ -941,6 +1067,29 @@ extern "C" int moe_gemm_gateup_swiglu_fwd(const uint16_t* xp, const uint16_t* w1
   a.n_tiles = (int)((I + Cfg::BN / 2 - 1) / (Cfg::BN / 2));
   a.m_slots = row_slots<Cfg>(R, E);
   return launch<GATEUP, Cfg, uint16_t>(a, (long long)a.n_tiles * a.m_slots, (hipStream_t)stream);
+}
+
+// Bytes of the blocked g/u buffer: one 4 KB record per 32 x 32 block of every row-tile slot the
+// tile list can have (ceil(R/256) + E bounds their number whatever the routing).
+extern "C" int64_t moe_gu_blocked_bytes(int64_t R, int64_t E, int64_t I) {
+  if (R <= 0 || E <= 0 || I <= 0) return 0;
+  using Cfg = CfgMain;
+  return (int64_t)row_slots<Cfg>(R, E) * (Cfg::BM / 32) * ((I + 31) / 32) * 4096;
+}
+
+extern "C" int moe_gemm_gateup_swiglu_fwd_blocked(const uint16_t* xp, const uint16_t* w1, const uint16_t* w3,
+                                                  const int32_t* offs, int64_t E, int64_t R, int64_t H,
+                                                  int64_t I, void* gu_blocked, uint16_t* act, void* stream) {
+  if (int rc = check_common(offs, E, R, H, I)) return rc;
+  if (R == 0) return 0;
+  MOE_CHECK_PTR(xp); MOE_CHECK_PTR(w1); MOE_CHECK_PTR(w3); MOE_CHECK_PTR(act); MOE_CHECK_PTR(gu_blocked);
+  using Cfg = CfgMain;
+  GemmArgs a{};
+  a.A0 = xp; a.B0 = w1; a.B1 = w3; a.C0 = gu_blocked; a.C2 = act; a.offs = offs;
+  a.E = (int)E; a.R = (int)R; a.N = (int)I; a.K = (int)H;
+  a.n_tiles = (int)((I + Cfg::BN / 2 - 1) / (Cfg::BN / 2));
+  a.m_slots = row_slots<Cfg>(R, E);
+  return launch<GATEUP, Cfg, uint16_t, true>(a, (long long)a.n_tiles * a.m_slots, (hipStream_t)stream);
 }
 
 extern "C" int moe_gemm_down_fwd(const uint16_t* act, const uint16_t* w2, const int32_t* offs,
@@ -994,6 +1143,25 @@ extern "C" int moe_gemm_dgrad_down_swiglu_bwd_dgate(const uint16_t* dyp, const u
                                                     float* dgate_part, void* stream) {
   if (R > 0 && !dgate_part) return MOE_ERR_NULL;
   return dgrad_down_impl(dyp, w2, g, u, offs, E, R, H, I, dg, du, dgate_part, stream);
+}
+
+extern "C" int moe_gemm_dgrad_down_swiglu_bwd_blocked(const uint16_t* dyp, const uint16_t* w2,
+                                                      const void* gu_blocked, const int32_t* offs, int64_t E,
+                                                      int64_t R, int64_t H, int64_t I, uint16_t* dg,
+                                                      uint16_t* du, int64_t ld_out, float* dgate_part,
+                                                      void* stream) {
+  if (int rc = check_common(offs, E, R, H, I)) return rc;
+  if (R == 0) return 0;
+  MOE_CHECK_PTR(dyp); MOE_CHECK_PTR(w2); MOE_CHECK_PTR(gu_blocked); MOE_CHECK_PTR(dg); MOE_CHECK_PTR(du);
+  if (ld_out != 0 && (ld_out < I || (ld_out % 8) != 0 || ld_out > (1 << 17))) return MOE_ERR_SHAPE;
+  using Cfg = CfgMain;
+  GemmArgs a{};
+  a.C2 = dgate_part;
+  a.A0 = dyp; a.B0 = w2; a.X0 = (const uint16_t*)gu_blocked; a.C0 = dg; a.C1 = du; a.offs = offs;
+  a.E = (int)E; a.R = (int)R; a.N = (int)I; a.K = (int)H; a.ld_c = (int)ld_out;
+  a.n_tiles = (int)((I + Cfg::BN - 1) / Cfg::BN);
+  a.m_slots = row_slots<Cfg>(R, E);
+  return launch<DGRAD_DOWN, Cfg, uint16_t, true>(a, (long long)a.n_tiles * a.m_slots, (hipStream_t)stream);
 }
 
 // The two row gradients side by side in one buffer: dgu [R, 2I], row = [dg row | du row].  The

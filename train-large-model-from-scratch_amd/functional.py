@@ -181,17 +181,27 @@ def _pair_ok(E, I, H, need_w, into, device):
     return (g1 is None) == (g3 is None) and (g1 is None or g1.dtype == g3.dtype) and p1.dtype == p3.dtype
 
 
-def _expert_backward(dyp, xp, g, u, act, w1b, w3b, w2b, offs, wdtype, need_w=(True, True, True),
+def _gateup(xp, w1b, w3b, offs, train: bool):
+    """Gate/up product and SwiGLU of the forward pass: -> (gu, act).  When a backward pass will
+    follow, g and u are saved in the library's blocked layout (read by nothing but the SwiGLU
+    backward); otherwise they are not written at all and `gu` is None."""
+    if train:
+        return ops.gemm_gateup_blocked(xp, w1b, w3b, offs)
+    return None, ops.gemm_gateup(xp, w1b, w3b, offs, save_gu=False)[2]
+
+
+def _expert_backward(dyp, xp, gu, act, w1b, w3b, w2b, offs, wdtype, need_w=(True, True, True),
                      into=None, gate_blocks=False):
-    """Shared backward of the expert FFN over expert-contiguous rows.  `need_w` and `into`
-    are per stack in the order gate, up, down.  With `gate_blocks` the fifth result holds the
-    per-row block sums of <dact, act> (the gate gradients are made from them), else None."""
+    """Shared backward of the expert FFN over expert-contiguous rows.  `gu` is the forward's g and
+    u in the library's blocked layout (ops.gemm_gateup_blocked).  `need_w` and `into` are per
+    stack in the order gate, up, down.  With `gate_blocks` the fifth result holds the per-row block
+    sums of <dact, act> (the gate gradients are made from them), else None."""
     E, I, H = w1b.shape
     into = into or (None, None, None)
     part = None
     if dyp.shape[0] > 0 and _pair_ok(E, I, H, need_w, into, dyp.device):
         # dg and du side by side: their two weight gradients are one grouped product
-        dgu, part = ops.gemm_dgrad_down_packed(dyp, w2b, g, u, offs, gate_blocks)
+        dgu, part = ops.gemm_dgrad_down_blocked(dyp, w2b, gu, offs, gate_blocks, packed=True)
         dxp = ops.gemm_dgrad_gateup_packed(dgu, w1b, w3b, offs)
         dw2 = _wgrad(dyp, act, offs, E, wdtype, need_w[2], into[2])
         p1, p3 = into[0], into[1]
@@ -204,10 +214,7 @@ def _expert_backward(dyp, xp, g, u, act, w1b, w3b, w2b, offs, wdtype, need_w=(Tr
             ops.gemm_wgrad_pair(dgu, xp, offs, E, p1.grad.dtype, out1=p1.grad, out3=p3.grad)
             dw1 = dw3 = None
         return dxp, dw1, dw3, dw2, part
-    if gate_blocks:
-        dg, du, part = ops.gemm_dgrad_down(dyp, w2b, g, u, offs, dgate_blocks=True)
-    else:
-        dg, du = ops.gemm_dgrad_down(dyp, w2b, g, u, offs)
+    dg, du, part = ops.gemm_dgrad_down_blocked(dyp, w2b, gu, offs, gate_blocks)
     dxp = ops.gemm_dgrad_gateup(dg, du, w1b, w3b, offs)
     segs = {}
     dw2 = _wgrad(dyp, act, offs, E, wdtype, need_w[2], into[2], segs)
@@ -230,11 +237,11 @@ class _MoEFFN(torch.autograd.Function):
         counts, offs, pos_to_row, row_to_pos = ops.histogram_scan(ids, E)
         xp = ops.permute_fwd(x, pos_to_row, k, row_to_pos)
         train = any(ctx.needs_input_grad)
-        g, u, act = ops.gemm_gateup(xp, w1b, w3b, offs, save_gu=train)
+        gu, act = _gateup(xp, w1b, w3b, offs, train)
         y = ops.gemm_down(act, w2b, offs)
         out = ops.combine_fwd(y, gates, row_to_pos, T, k, x.dtype)
         if train:  # (y is not kept: the gate gradients come out of the dgrad-down kernel)
-            ctx.save_for_backward(xp, g, u, act, gates, ids, offs, pos_to_row, row_to_pos,
+            ctx.save_for_backward(xp, gu, act, gates, ids, offs, pos_to_row, row_to_pos,
                                   w1b, w3b, w2b)
         ctx.k, ctx.E = k, E
         ctx.grad_params = grad_params
@@ -246,7 +253,7 @@ class _MoEFFN(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dout, *unused):
-        xp, g, u, act, gates, ids, offs, pos_to_row, row_to_pos, w1b, w3b, w2b = ctx.saved_tensors
+        xp, gu, act, gates, ids, offs, pos_to_row, row_to_pos, w1b, w3b, w2b = ctx.saved_tensors
         k, E = ctx.k, ctx.E
         if dout is None:
             dout = torch.zeros(ctx.out_shape, dtype=ctx.x_dtype, device=xp.device)
@@ -255,7 +262,7 @@ class _MoEFFN(torch.autograd.Function):
         if dout.dtype not in (torch.bfloat16, torch.float32):
             dout = dout.float()
         dyp, _ = ops.combine_bwd(dout, None, gates, pos_to_row, k, row_to_pos)
-        dxp, dw1, dw3, dw2, part = _expert_backward(dyp, xp, g, u, act, w1b, w3b, w2b, offs, ctx.w_dtype,
+        dxp, dw1, dw3, dw2, part = _expert_backward(dyp, xp, gu, act, w1b, w3b, w2b, offs, ctx.w_dtype,
                                                     ctx.needs_input_grad[2:5], ctx.grad_params,
                                                     ctx.needs_input_grad[1] or ctx.needs_input_grad[6])
         dx = ops.permute_bwd(dxp, row_to_pos, T, k, ctx.x_dtype) if ctx.needs_input_grad[0] else None
@@ -331,7 +338,7 @@ class _PreNormMoE(torch.autograd.Function):
         counts, offs, pos_to_row, row_to_pos = ops.histogram_scan(ids, E)
         xp = ops.permute_fwd(xn, pos_to_row, k, row_to_pos)
         train = any(ctx.needs_input_grad)
-        g, u, act = ops.gemm_gateup(xp, w1b, w3b, offs, save_gu=train)
+        gu, act = _gateup(xp, w1b, w3b, offs, train)
         y = ops.gemm_down(act, w2b, offs)
         if add_residual:
             out = ops.combine_fwd_residual(y, gates, row_to_pos, x, k)
@@ -339,7 +346,7 @@ class _PreNormMoE(torch.autograd.Function):
             out = ops.combine_fwd(y, gates, row_to_pos, T, k, x.dtype)
         ctx.has_norm = norm_w is not None
         if train:
-            ctx.save_for_backward(x if ctx.has_norm else None, nw, rstd, xn, wrb, xp, g, u, act, gates, ids,
+            ctx.save_for_backward(x if ctx.has_norm else None, nw, rstd, xn, wrb, xp, gu, act, gates, ids,
                                   offs, pos_to_row, row_to_pos, w1b, w3b, w2b)
         ctx.k, ctx.E, ctx.add_residual = k, E, add_residual
         ctx.grad_params = grad_params
@@ -352,7 +359,7 @@ class _PreNormMoE(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dout, dlogits_ext, *unused):
-        (x, nw, rstd, xn, wrb, xp, g, u, act, gates, ids, offs, pos_to_row, row_to_pos,
+        (x, nw, rstd, xn, wrb, xp, gu, act, gates, ids, offs, pos_to_row, row_to_pos,
          w1b, w3b, w2b) = ctx.saved_tensors
         k, E = ctx.k, ctx.E
         T = ctx.x_shape[0]
@@ -362,7 +369,7 @@ class _PreNormMoE(torch.autograd.Function):
         if dout.dtype != ctx.x_dtype:
             dout = dout.to(ctx.x_dtype)
         dyp, _ = ops.combine_bwd(dout, None, gates, pos_to_row, k, row_to_pos)
-        dxp, dw1, dw3, dw2, part = _expert_backward(dyp, xp, g, u, act, w1b, w3b, w2b, offs, ctx.w_dtype,
+        dxp, dw1, dw3, dw2, part = _expert_backward(dyp, xp, gu, act, w1b, w3b, w2b, offs, ctx.w_dtype,
                                                     ctx.needs_input_grad[3:6], ctx.grad_params, True)
         dgates = ops.dgates_from_blocks(part, gates, row_to_pos, pos_to_row)
         dbias = None
@@ -447,11 +454,11 @@ class _ExpertsRows(torch.autograd.Function):
         counts, offs, pos_to_row, row_to_pos, bad = ops.histogram_scan(ids32, E, return_bad=True)
         xp = ops.permute_fwd(rows, pos_to_row, 1)
         train = any(ctx.needs_input_grad)
-        g, u, act = ops.gemm_gateup(xp, w1b, w3b, offs, save_gu=train)
+        gu, act = _gateup(xp, w1b, w3b, offs, train)
         y = ops.gemm_down(act, w2b, offs)
         out = ops.combine_fwd(y, None, row_to_pos, R, 1, rows.dtype)
         if train:
-            ctx.save_for_backward(xp, g, u, act, offs, pos_to_row, row_to_pos, w1b, w3b, w2b)
+            ctx.save_for_backward(xp, gu, act, offs, pos_to_row, row_to_pos, w1b, w3b, w2b)
         ctx.x_dtype, ctx.w_dtype = rows.dtype, w1.dtype
         ctx.grad_params = grad_params
         ctx.mark_non_differentiable(counts, offs, pos_to_row, row_to_pos, bad)
@@ -461,7 +468,7 @@ class _ExpertsRows(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dout, *unused):
-        xp, g, u, act, offs, pos_to_row, row_to_pos, w1b, w3b, w2b = ctx.saved_tensors
+        xp, gu, act, offs, pos_to_row, row_to_pos, w1b, w3b, w2b = ctx.saved_tensors
         if dout is None:
             dout = torch.zeros(ctx.out_shape, dtype=ctx.x_dtype, device=xp.device)
         R = dout.shape[0]
@@ -469,7 +476,7 @@ class _ExpertsRows(torch.autograd.Function):
         if dout.dtype not in (torch.bfloat16, torch.float32):
             dout = dout.float()
         dyp, _ = ops.combine_bwd(dout, None, None, pos_to_row, 1)
-        dxp, dw1, dw3, dw2, _ = _expert_backward(dyp, xp, g, u, act, w1b, w3b, w2b, offs,
+        dxp, dw1, dw3, dw2, _ = _expert_backward(dyp, xp, gu, act, w1b, w3b, w2b, offs,
                                                  ctx.w_dtype, ctx.needs_input_grad[2:5], ctx.grad_params)
         drows = ops.permute_bwd(dxp, row_to_pos, R, 1, ctx.x_dtype) if ctx.needs_input_grad[0] else None
         return drows, None, dw1, dw3, dw2, None

@@ -25,6 +25,10 @@ SIGNATURES = {
     "moe_permute_bwd": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp, _int, _vp]),
     "moe_permute_bwd_addend": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _i64, _vp, _int, _vp]),
     "moe_gemm_gateup_swiglu_fwd": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp]),
+    "moe_gu_blocked_bytes": (_i64, [_i64, _i64, _i64]),
+    "moe_gemm_gateup_swiglu_fwd_blocked": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _vp]),
+    "moe_gemm_dgrad_down_swiglu_bwd_blocked": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _i64,
+                                                      _vp, _vp]),
     "moe_gemm_down_fwd": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp]),
     "moe_gemm_dgrad_down_swiglu_bwd": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _vp]),
     "moe_dgate_blocks": (_i64, [_i64]),

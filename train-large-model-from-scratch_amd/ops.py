@@ -126,6 +126,42 @@ def gemm_gateup(xp, w1, w3, offs, save_gu: bool):
     return g, u, act
 
 
+def gemm_gateup_blocked(xp, w1, w3, offs):
+    """gemm_gateup for a forward pass whose g and u only the SwiGLU backward will read: they are
+    left in the library's blocked layout (an opaque uint8 buffer; see include/moe_gfx950.h), which
+    the forward kernel writes straight from its registers.  -> gu_blocked, act [R,I]."""
+    R, H = xp.shape
+    E, I, _ = w1.shape
+    L = _lib.load()
+    act = torch.empty(R, I, dtype=torch.bfloat16, device=xp.device)
+    gu = torch.empty(max(L.cdll.moe_gu_blocked_bytes(R, E, I), 16), dtype=torch.uint8, device=xp.device)
+    L.call("moe_gemm_gateup_swiglu_fwd_blocked", _p(xp), _p(w1), _p(w3), _p(offs), E, R, H, I, _p(gu), _p(act),
+           _stream())
+    return gu, act
+
+
+def gemm_dgrad_down_blocked(dyp, w2, gu, offs, dgate_blocks: bool = False, packed: bool = False):
+    """gemm_dgrad_down / gemm_dgrad_down_packed on blocked g/u: -> (dg, du, part) with `dg`, `du` [R,I], or
+    (dgu, part) with dgu [R,2I] = [dg | du] when `packed`; `part` as in gemm_dgrad_down (None without
+    `dgate_blocks`).  Same bits as the row-major entries."""
+    R, H = dyp.shape
+    E, _, I = w2.shape
+    L = _lib.load()
+    part = torch.empty(L.cdll.moe_dgate_blocks(I), R, dtype=torch.float32, device=dyp.device) if dgate_blocks else None
+    if packed:
+        dgu = torch.empty(R, 2 * I, dtype=torch.bfloat16, device=dyp.device)
+        dg, du, ld = dgu, dgu[:, I:], 2 * I
+    else:
+        dg = torch.empty(R, I, dtype=torch.bfloat16, device=dyp.device)
+        du = torch.empty_like(dg)
+        ld = 0
+    L.call("moe_gemm_dgrad_down_swiglu_bwd_blocked", _p(dyp), _p(w2), _p(gu), _p(offs), E, R, H, I,
+           dg.data_ptr(), du.data_ptr(), ld, _p(part), _stream())
+    if packed:
+        return dgu, part
+    return dg, du, part
+
+
 def gemm_down(act, w2, offs):
     R, I = act.shape
     E, H, _ = w2.shape
