@@ -59,6 +59,78 @@ def _event_time_ms(torch, fn, iters, warmup):
     return s.elapsed_time(e) / iters
 
 
+def _timed_steps(torch, step, steps, warmup):
+    """W untimed steps, then K steps bracketed by synchronisations: -> (wall-clock mean ms per step,
+    HIP-event median, HIP-event minimum).  One event is recorded on the launch stream after every
+    step (K+1 records in all), so that the spread over the steps is seen next to the mean."""
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    t0 = time.perf_counter()
+    marks[0].record()
+    for i in range(steps):
+        step()
+        marks[i + 1].record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3 / steps
+    per = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(steps))
+    median = per[len(per) // 2] if len(per) % 2 else 0.5 * (per[len(per) // 2 - 1] + per[len(per) // 2])
+    return wall, median, per[0]
+
+
+# flops of one launch of each GEMM entry point, in units of R*H*I
+_GEMM_RHI = {"moe_gemm_gateup_swiglu_fwd": 4, "moe_gemm_gateup_swiglu_fwd_blocked": 4,
+             "moe_gemm_down_fwd": 2, "moe_gemm_dgrad_down_swiglu_bwd": 2,
+             "moe_gemm_dgrad_down_swiglu_bwd_dgate": 2, "moe_gemm_dgrad_down_swiglu_bwd_packed": 2,
+             "moe_gemm_dgrad_down_swiglu_bwd_blocked": 2,
+             "moe_gemm_dgrad_gateup": 4, "moe_gemm_dgrad_gateup_packed": 4, "moe_gemm_wgrad_pair": 4,
+             "moe_gemm_wgrad": 2}
+
+
+def _launches_in_step(torch, P, step, steps, RHI, flops):
+    """The same K steps once more with a pair of HIP events around every launch of the library
+    (its `observer` hook): -> (records per launch in step order, roofline fields of the GEMM launch
+    with the largest duration, ms per step of this instrumented region)."""
+    watch = _LaunchEvents(torch)
+    P.lib.load().observer = watch
+    t0 = time.perf_counter()
+    try:
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+    finally:
+        P.lib.load().observer = None
+    ms_events = (time.perf_counter() - t0) * 1e3 / steps
+    in_step = watch.per_launch_ms(steps)
+    recs = []
+    # moe_gemm_wgrad also serves the router's small split-k product, and (with few experts) the
+    # row segments of one stack: a launch counts as an expert weight gradient of 2*R*H*I when it
+    # lasts at least a tenth of the longest one
+    longest_wgrad = max([m for n, m in in_step if n == "moe_gemm_wgrad"], default=0.0)
+    for name, kms in in_step:
+        rec = {"entry": name, "ms": round(kms, 4)}
+        f = _GEMM_RHI.get(name)
+        if f and kms > 0 and not (name == "moe_gemm_wgrad" and kms < 0.1 * longest_wgrad):
+            rec.update(achieved=round(f * RHI / kms / 1e9, 1), unit="TFLOP/s",
+                       frac=round(f * RHI / kms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4))
+        recs.append(rec)
+    roof = None
+    g_in = [r for r in recs if "frac" in r]
+    if g_in:
+        dom = max(g_in, key=lambda r: r["ms"])
+        g_ms = sum(r["ms"] for r in g_in)
+        roof = {"kernel": dom["entry"].replace("moe_", "", 1), "bound": "mfma", "achieved": dom["achieved"],
+                "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": dom["frac"], "traffic": None,
+                "ms": dom["ms"],
+                "measured": f"HIP events around this launch in each of {steps} steps that follow the timed "
+                            f"ones ({round(ms_events, 4)} ms per step with the events)",
+                "all_gemms_tflops": round(flops / g_ms / 1e9, 1),
+                "all_gemms_frac": round(flops / g_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
+                "launches_ms_sum": round(sum(r["ms"] for r in recs), 4)}
+    return recs, roof, ms_events
+
+
 class _LaunchEvents:
     """Observer of the library's launches: a pair of HIP events around every entry point,
     recorded on torch's current stream (the stream the launch is handed), so that each kernel's
@@ -233,24 +305,22 @@ def time_layer_config(P, torch, dev, cfg_id, steps, warmup):
             out, _ = P.routed_moe(x, wr, *ws, s.k, bias=bias)
             if s.backward:
                 out.backward(dy)
-    for _ in range(warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        step()
-    torch.cuda.synchronize()
-    ms = (time.perf_counter() - t0) * 1e3 / steps
+    ms, ms_median, ms_min = _timed_steps(torch, step, steps, warmup)
     flops = P.configs.gemm_flops(s)
+    recs, roof, _ = _launches_in_step(torch, P, step, steps, s.R * s.H * s.I, flops)
     return {"config": cfg_id, "workload": s.name, "entry": "experts_rows" if s.rows_entry else "routed_moe",
-            "ms_per_step": round(ms, 4), "tflops": round(flops / ms / 1e9, 1),
+            "ms_per_step": round(ms, 4), "ms_per_step_median": round(ms_median, 4), "ms_per_step_min": round(ms_min, 4),
+            "tflops": round(flops / ms / 1e9, 1),
             "mfma_peak_frac": round(flops / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
-            "tokens_per_s": round(s.T / (ms * 1e-3), 1), "steps": steps}
+            "tokens_per_s": round(s.T / (ms * 1e-3), 1), "steps": steps, "roofline": roof,
+            "kernels_in_step": recs}
 
 
 def cpu_leg(P, torch, cfg_id, fraction=1.0):
     """The oracle's per-expert loop (forward, and backward where the configuration has one) on
-    the host cores: the CPU baseline of a configuration."""
+    the host cores: the CPU baseline of a configuration.  The two small configurations are run
+    once to warm up and then three times (the median is reported); the large ones, which take
+    seconds, once."""
     from oracle import moe_oracle as O
     ncores = os.cpu_count() or 1
     ncores = min(ncores, int(os.environ.get("OMP_NUM_THREADS", ncores)))
@@ -258,24 +328,37 @@ def cpu_leg(P, torch, cfg_id, fraction=1.0):
     cin = P.configs.make_inputs(cfg_id, scale_tokens=fraction)
     s = cin["shape"]
     w32 = [cin[n].float() for n in ("w1", "w3", "w2")]
-    t0 = time.perf_counter()
+
+    def one_pass():
+        t0 = time.perf_counter()
+        if s.rows_entry:
+            f = O.experts_rows_forward(cin["x"], cin["ids"].numpy(), *w32)
+            O.experts_rows_backward(f, cin["dy"].float(), *w32)
+        else:
+            wr32 = cin["wr"].float()
+            f = O.moe_forward(cin["x"], wr32, *w32, s.k, bias=cin.get("bias"), logits_dtype=torch.bfloat16)
+            if s.backward:
+                O.moe_backward(f, cin["dy"].float(), wr32, *w32)
+        return time.perf_counter() - t0
+
     if s.rows_entry:
-        f = O.experts_rows_forward(cin["x"], cin["ids"].numpy(), *w32)
-        O.experts_rows_backward(f, cin["dy"].float(), *w32)
         rows = cin["x"].shape[0]
         toks = rows / s.k
     else:
-        wr32 = cin["wr"].float()
-        f = O.moe_forward(cin["x"], wr32, *w32, s.k, bias=cin.get("bias"), logits_dtype=torch.bfloat16)
-        if s.backward:
-            O.moe_backward(f, cin["dy"].float(), wr32, *w32)
         toks = cin["x"].shape[0]
         rows = toks * s.k
-    dt = time.perf_counter() - t0
+    small = cfg_id in (1, 2)
+    if small:
+        one_pass()
+        times = sorted(one_pass() for _ in range(3))
+        dt, how = times[1], f"one warm-up pass, then the median of three timed passes ({times[1]:.3f} s)"
+    else:
+        dt = one_pass()
+        how = f"one timed pass of {dt:.2f} s"
     cflops = (18 if s.backward else 6) * rows * s.H * s.I
     return {"value": round(cflops / dt / 1e12, 4), "unit": "TFLOP/s", "cores": ncores, "kind": "port",
             "sample": f"oracle per-expert loop, fp32 math on the same bf16 inputs, {int(toks)} of {s.T} tokens "
-                      f"({rows} routed rows, all {s.E} experts), one timed pass of {dt:.2f} s",
+                      f"({rows} routed rows, all {s.E} experts), {how}",
             "tokens_per_s": round(toks / dt, 1)}
 
 
@@ -397,30 +480,16 @@ def main():
             if s.backward:
                 out.backward(dy)
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms, ms_median, ms_min = _timed_steps(torch, step, args.steps, args.warmup)
     tflops = flops / ms / 1e9
     # The same K steps once more, now with a pair of HIP events around every launch: each
     # kernel's duration inside the step.  A region of its own because the 2 x 15 event records
-    # per step cost about 1 % of the step (5.33 against 5.28 ms), which the headline figure
-    # should not carry; only where the step is bound by the GPU (the two large configurations).
-    in_step, ms_events = [], None
-    if args.kernel_events and args.config in (3, 4):
-        watch = _LaunchEvents(torch)
-        P.lib.load().observer = watch
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            step()
-        torch.cuda.synchronize()
-        ms_events = (time.perf_counter() - t0) * 1e3 / args.steps
-        P.lib.load().observer = None
-        in_step = watch.per_launch_ms(args.steps)
+    # per step cost about 1 % of the step (5.33 against 5.28 ms on configuration 3), which the
+    # headline figure should not carry.  (Where the step is bound by the host's launches, the two
+    # small configurations, the events lengthen the step but not the kernels they bracket.)
+    in_step_recs, roof_in_step, ms_events = [], None, None
+    if args.kernel_events:
+        in_step_recs, roof_in_step, ms_events = _launches_in_step(torch, P, step, args.steps, RHI, flops)
     tokens_per_s = s.T / (ms * 1e-3)
 
     # the same step captured once in a HIP graph and replayed: what a caller gets who removes
@@ -513,6 +582,12 @@ def main():
             w_master = torch.empty(w1.shape, dtype=torch.float32, device=dev).normal_()
             kernels.append(("cast_f32_bf16_one_weight_stack", lambda: ops.cast_bf16(w_master), 0,
                             w_master.numel() * 6, 0))
+            # what the memory system of this part gives plain streaming kernels of the runtime, in the
+            # same run: the yardstick for the row movers (a 1 GiB device copy, a 1 GiB fill)
+            src_c = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+            dst_c = torch.empty_like(src_c)
+            kernels.append(("reference_device_copy_1GiB", lambda: dst_c.copy_(src_c), 0, 2 * src_c.numel() * 4, 0))
+            kernels.append(("reference_device_fill_1GiB", lambda: dst_c.zero_(), 0, src_c.numel() * 4, 0))
             per_kernel = []
             for name, fn, fl, by, launches in kernels:
                 kms = _event_time_ms(torch, fn, 10, 2)
@@ -524,6 +599,7 @@ def main():
                     rec.update(bound="hbm", achieved=round(by / kms / 1e6, 1), unit="GB/s",
                                frac=round(by / kms / 1e6 / HBM_PEAK_GBS, 4))
                 per_kernel.append(rec)
+            del src_c, dst_c
             # what the vendor's dense GEMM library reaches on this part on problems of the same size
             # with none of the layer's structure (one weight for all rows, no ragged groups, no fused
             # epilogue, one output): the practical ceiling the grouped kernels are measured against
@@ -554,41 +630,14 @@ def main():
     # the same kernels inside the timed steps (events around every launch): these are the
     # durations the roofline object reports where they exist; the figures from the separate
     # loops above stay beside them
-    in_step_recs = []
-    if in_step:
-        gemm_flops_of = {"moe_gemm_gateup_swiglu_fwd": 4, "moe_gemm_gateup_swiglu_fwd_blocked": 4,
-                         "moe_gemm_dgrad_down_swiglu_bwd_blocked": 2,
-                         "moe_gemm_down_fwd": 2, "moe_gemm_dgrad_down_swiglu_bwd": 2,
-                         "moe_gemm_dgrad_down_swiglu_bwd_dgate": 2, "moe_gemm_dgrad_down_swiglu_bwd_packed": 2,
-                         "moe_gemm_dgrad_gateup": 4, "moe_gemm_dgrad_gateup_packed": 4, "moe_gemm_wgrad_pair": 4,
-                         "moe_gemm_wgrad": 2}
-        # moe_gemm_wgrad also serves the router's small split-k product: only launches of at least a
-        # tenth of the longest one are the experts' weight gradients
-        longest_wgrad = max([m for n, m in in_step if n == "moe_gemm_wgrad"], default=0.0)
-        for name, kms in in_step:
-            rec = {"entry": name, "ms": round(kms, 4)}
-            f = gemm_flops_of.get(name)
-            if f and not (name == "moe_gemm_wgrad" and kms < 0.1 * longest_wgrad):
-                rec.update(achieved=round(f * RHI / kms / 1e9, 1), unit="TFLOP/s",
-                           frac=round(f * RHI / kms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4))
-            in_step_recs.append(rec)
-        g_in = [r for r in in_step_recs if "frac" in r]
-        if g_in:
-            dom = max(g_in, key=lambda r: r["ms"])
-            g_ms = sum(r["ms"] for r in g_in)
-            roofline.update(
-                kernel=dom["entry"].replace("moe_", "", 1), achieved=dom["achieved"], frac=dom["frac"],
-                ms=dom["ms"],
-                measured=f"HIP events around this launch in each of {args.steps} steps that follow the timed "
-                         f"ones ({round(ms_events, 4)} ms per step with the events)",
-                achieved_back_to_back=dominant["achieved"] if dominant else None,
-                all_gemms_tflops=round(flops / g_ms / 1e9, 1),
-                all_gemms_frac=round(flops / g_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
-                launches_ms_sum=round(sum(r["ms"] for r in in_step_recs), 4))
+    if roof_in_step:
+        roofline.update(roof_in_step)
+        roofline["achieved_back_to_back"] = dominant["achieved"] if dominant else None
 
     roofline["traffic"] = MEASURED_HBM_BYTES_PER_LAUNCH.get((args.config, roofline["kernel"]))
     roofline["traffic_source"] = ("rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this benchmark, "
-                                  "profiles/grouped_gemm_cfg3_pmc.txt (not measured by this run)")
+                                  "profiles/grouped_gemm_cfg3_pmc.txt (not measured by this run)"
+                                  if roofline["traffic"] is not None else None)
 
     # ---------------- CPU baseline: the oracle's per-expert loop on a bounded sample
     cpu = None if args.no_cpu else cpu_leg(P, torch, args.config, args.cpu_fraction)
@@ -616,6 +665,9 @@ def main():
         "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
+        "ms_per_step_median": round(ms_median, 4), "ms_per_step_min": round(ms_min, 4),
+        "ms_per_step_timing": "ms_per_step: wall clock around the K steps between two synchronisations, / K; "
+                              "median and min: HIP events recorded on the launch stream after every step",
         "config": {"workload": s.name, "tokens": s.T, "hidden": s.H, "experts": s.E, "top_k": s.k,
                    "ffn": s.I, "routed_rows": s.R, "gemm_flops_per_step": flops},
         "tokens_per_s": round(tokens_per_s, 1),

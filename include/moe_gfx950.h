@@ -192,6 +192,15 @@ int moe_gemm_dgrad_down_swiglu_bwd_blocked(const uint16_t* dyp, const uint16_t* 
                                            int64_t R, int64_t H, int64_t I, uint16_t* dg,
                                            uint16_t* du, int64_t ld_out, float* dgate_part,
                                            void* stream);
+/* Test hook (no counterpart in the reference).  The four row-ragged products (gate/up, down and
+ * their two input gradients) run on 256-row tiles, or on 128-row tiles when the launch has too few
+ * large tiles for half of the compute units; the choice is made from R, E and the
+ * output width alone.  moe_gemm_force_row_tile(128 or 256) forces one of them for every later
+ * call, 0 restores the automatic choice; the previous setting is returned.  Process-wide and not
+ * synchronised with calls in flight on other host threads.  No result depends on the choice:
+ * every output element is accumulated over k in the same order on both tile heights, so all
+ * outputs (the gate gradients' block sums included) are the same bits either way. */
+int moe_gemm_force_row_tile(int rows);
 /* Backward of gate/up w.r.t. the rows (autograd of mlp.py:154-155): dxp = dg*W1 + du*W3. */
 int moe_gemm_dgrad_gateup(const uint16_t* dg, const uint16_t* du, const uint16_t* w1,
                           const uint16_t* w3, const int32_t* offs, int64_t E, int64_t R,

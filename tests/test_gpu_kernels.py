@@ -404,6 +404,24 @@ def test_expert_gemms_forward_backward(ops, R, H, I, E, empty):
     assert torch.equal(dgu_b[:, :I], dg) and torch.equal(dgu_b[:, I:], du)
     assert torch.equal(part_b3.view(torch.int32), part_r.view(torch.int32))
     dxp = ops.gemm_dgrad_gateup(dg, du, w1.cuda(), w3.cuda(), offs)
+    # both row-tile heights of the four row-ragged products, forced in turn (the automatic choice
+    # above took one of them from the shape): the same bits on every output
+    L = ops._lib.load()
+    try:
+        for rows in (128, 256):
+            L.cdll.moe_gemm_force_row_tile(rows)
+            g_t, u_t, act_t = ops.gemm_gateup(xp.cuda(), w1.cuda(), w3.cuda(), offs, save_gu=True)
+            assert torch.equal(g_t, g) and torch.equal(u_t, u) and torch.equal(act_t, act), rows
+            assert torch.equal(ops.gemm_down(act, w2.cuda(), offs), y), rows
+            gu_t, act_t = ops.gemm_gateup_blocked(xp.cuda(), w1.cuda(), w3.cuda(), offs)
+            dg_t, du_t, part_t = ops.gemm_dgrad_down_blocked(dyp.cuda(), w2.cuda(), gu_t, offs, dgate_blocks=True)
+            assert torch.equal(act_t, act) and torch.equal(dg_t, dg) and torch.equal(du_t, du), rows
+            assert torch.equal(part_t.view(torch.int32), part_r.view(torch.int32)), rows
+            dg_t, du_t = ops.gemm_dgrad_down(dyp.cuda(), w2.cuda(), g, u, offs)
+            assert torch.equal(dg_t, dg) and torch.equal(du_t, du), rows
+            assert torch.equal(ops.gemm_dgrad_gateup(dg, du, w1.cuda(), w3.cuda(), offs), dxp), rows
+    finally:
+        L.cdll.moe_gemm_force_row_tile(0)
     dgf, duf = dg.float().cpu(), du.float().cpu()
     ref_dxp = torch.zeros(R, H)
     ref_dw1, ref_dw3 = torch.zeros(E, I, H), torch.zeros(E, I, H)

@@ -803,6 +803,9 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WAVES_PER_SIMD) void grouped_gemm_ker
             }
             put4(0, j, q, dg[0], dg[1], dg[2], dg[3]);
             put4(1, j, q, du[0], du[1], du[2], du[3]);
+            // (the running sum is wanted here, not at the end of the strip: left alone the compiler
+            // may defer its chain of additions and keep every du and u alive for it)
+            asm volatile("" : "+v"(rowdot));
           }
           __builtin_amdgcn_sched_barrier(0);  // (the loads must not move up: their registers are in use)
           if (i + 1 < FM) request_block(i + 1, j, blk_in);
@@ -843,6 +846,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WAVES_PER_SIMD) void grouped_gemm_ker
             }
             put4(0, j, q, dg[0], dg[1], dg[2], dg[3]);
             put4(1, j, q, du[0], du[1], du[2], du[3]);
+            asm volatile("" : "+v"(rowdot));  // (summed here: see the blocked variant above)
           }
         {
           // One partial per 64-column block and row (block-major, so that a wave writes 32
@@ -1000,6 +1004,10 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WAVES_PER_SIMD) void grouped_gemm_ker
 #define MOE_WN 4
 #endif
 using CfgMain = TileCfg<MOE_BM, MOE_BN, MOE_BK, MOE_WM, MOE_WN>;
+// Row tiles of half the height (the eight waves 64 x 64 each) for launches too small to give even
+// half of the compute units one of the large tiles: twice the tiles, each at about 0.7 of the
+// large tile's cost, spread such a launch over twice the compute units.
+using CfgSmall = TileCfg<MOE_BM / 2, MOE_BN, MOE_BK, MOE_WM, MOE_WN>;
 
 int compute_units() {
   static int cus[MOE_MAX_DEVICES];  // per GPU; 0 = not asked yet
@@ -1050,6 +1058,22 @@ int row_slots(int64_t R, int64_t E) {
   return (int)((R + Cfg::BM - 1) / Cfg::BM + E);
 }
 
+// Which row-tile height a row-ragged launch uses: decided from the shapes alone (never from the
+// routing: no host synchronisation), the same way for the forward kernel that writes blocked g/u
+// and the backward kernel that reads it (both pass I as `cols`).  Measured on the two small
+// benchmark configurations: 4096 rows of 8 experts (48 large tiles by this count) run 24 % faster
+// on the small tiles, 16384 rows (144) no faster.  `forced_row_tile` (0: automatic) is a test hook.
+int forced_row_tile = 0;
+bool small_row_tiles(int64_t R, int64_t E, int64_t cols) {
+  if (forced_row_tile) return forced_row_tile == CfgSmall::BM;
+  const int64_t tiles = (int64_t)row_slots<CfgMain>(R, E) * ((cols + CfgMain::BN - 1) / CfgMain::BN);
+  return 2 * tiles < (int64_t)compute_units();
+}
+template <typename F>
+int with_row_tile(bool small, F&& f) {
+  return small ? f(CfgSmall{}) : f(CfgMain{});
+}
+
 }  // namespace
 
 extern "C" int moe_gemm_gateup_swiglu_fwd(const uint16_t* xp, const uint16_t* w1, const uint16_t* w3,
@@ -1060,13 +1084,15 @@ extern "C" int moe_gemm_gateup_swiglu_fwd(const uint16_t* xp, const uint16_t* w1
   if (R == 0) return 0;
   MOE_CHECK_PTR(xp); MOE_CHECK_PTR(w1); MOE_CHECK_PTR(w3); MOE_CHECK_PTR(act);
   if ((g == nullptr) != (u == nullptr)) return MOE_ERR_NULL;
-  using Cfg = CfgMain;
-  GemmArgs a{};
-  a.A0 = xp; a.B0 = w1; a.B1 = w3; a.C0 = g; a.C1 = u; a.C2 = act; a.offs = offs;
-  a.E = (int)E; a.R = (int)R; a.N = (int)I; a.K = (int)H;
-  a.n_tiles = (int)((I + Cfg::BN / 2 - 1) / (Cfg::BN / 2));
-  a.m_slots = row_slots<Cfg>(R, E);
-  return launch<GATEUP, Cfg, uint16_t>(a, (long long)a.n_tiles * a.m_slots, (hipStream_t)stream);
+  return with_row_tile(small_row_tiles(R, E, I), [&](auto cfg) {
+    using Cfg = decltype(cfg);
+    GemmArgs a{};
+    a.A0 = xp; a.B0 = w1; a.B1 = w3; a.C0 = g; a.C1 = u; a.C2 = act; a.offs = offs;
+    a.E = (int)E; a.R = (int)R; a.N = (int)I; a.K = (int)H;
+    a.n_tiles = (int)((I + Cfg::BN / 2 - 1) / (Cfg::BN / 2));
+    a.m_slots = row_slots<Cfg>(R, E);
+    return launch<GATEUP, Cfg, uint16_t>(a, (long long)a.n_tiles * a.m_slots, (hipStream_t)stream);
+  });
 }
 
 // Bytes of the blocked g/u buffer: one 4 KB record per 32 x 32 block of every row-tile slot the
@@ -1083,13 +1109,15 @@ extern "C" int moe_gemm_gateup_swiglu_fwd_blocked(const uint16_t* xp, const uint
   if (int rc = check_common(offs, E, R, H, I)) return rc;
   if (R == 0) return 0;
   MOE_CHECK_PTR(xp); MOE_CHECK_PTR(w1); MOE_CHECK_PTR(w3); MOE_CHECK_PTR(act); MOE_CHECK_PTR(gu_blocked);
-  using Cfg = CfgMain;
-  GemmArgs a{};
-  a.A0 = xp; a.B0 = w1; a.B1 = w3; a.C0 = gu_blocked; a.C2 = act; a.offs = offs;
-  a.E = (int)E; a.R = (int)R; a.N = (int)I; a.K = (int)H;
-  a.n_tiles = (int)((I + Cfg::BN / 2 - 1) / (Cfg::BN / 2));
-  a.m_slots = row_slots<Cfg>(R, E);
-  return launch<GATEUP, Cfg, uint16_t, true>(a, (long long)a.n_tiles * a.m_slots, (hipStream_t)stream);
+  return with_row_tile(small_row_tiles(R, E, I), [&](auto cfg) {
+    using Cfg = decltype(cfg);
+    GemmArgs a{};
+    a.A0 = xp; a.B0 = w1; a.B1 = w3; a.C0 = gu_blocked; a.C2 = act; a.offs = offs;
+    a.E = (int)E; a.R = (int)R; a.N = (int)I; a.K = (int)H;
+    a.n_tiles = (int)((I + Cfg::BN / 2 - 1) / (Cfg::BN / 2));
+    a.m_slots = row_slots<Cfg>(R, E);
+    return launch<GATEUP, Cfg, uint16_t, true>(a, (long long)a.n_tiles * a.m_slots, (hipStream_t)stream);
+  });
 }
 
 extern "C" int moe_gemm_down_fwd(const uint16_t* act, const uint16_t* w2, const int32_t* offs,
@@ -1098,13 +1126,24 @@ extern "C" int moe_gemm_down_fwd(const uint16_t* act, const uint16_t* w2, const 
   if (int rc = check_common(offs, E, R, H, I)) return rc;
   if (R == 0) return 0;
   MOE_CHECK_PTR(act); MOE_CHECK_PTR(w2); MOE_CHECK_PTR(y);
-  using Cfg = CfgMain;
-  GemmArgs a{};
-  a.A0 = act; a.B0 = w2; a.C0 = y; a.offs = offs;
-  a.E = (int)E; a.R = (int)R; a.N = (int)H; a.K = (int)I;
-  a.n_tiles = (int)((H + Cfg::BN - 1) / Cfg::BN);
-  a.m_slots = row_slots<Cfg>(R, E);
-  return launch<DOWN, Cfg, uint16_t>(a, (long long)a.n_tiles * a.m_slots, (hipStream_t)stream);
+  return with_row_tile(small_row_tiles(R, E, H), [&](auto cfg) {
+    using Cfg = decltype(cfg);
+    GemmArgs a{};
+    a.A0 = act; a.B0 = w2; a.C0 = y; a.offs = offs;
+    a.E = (int)E; a.R = (int)R; a.N = (int)H; a.K = (int)I;
+    a.n_tiles = (int)((H + Cfg::BN - 1) / Cfg::BN);
+    a.m_slots = row_slots<Cfg>(R, E);
+    return launch<DOWN, Cfg, uint16_t>(a, (long long)a.n_tiles * a.m_slots, (hipStream_t)stream);
+  });
+}
+
+// Test hook: 0 lets every row-ragged launch choose its row-tile height (the default), 128 or 256
+// forces it.  Process-wide and not synchronised: for tests that want every shape on every tile
+// configuration, not for production callers.  Returns the previous setting.
+extern "C" int moe_gemm_force_row_tile(int rows) {
+  const int before = forced_row_tile;
+  if (rows == 0 || rows == CfgSmall::BM || rows == CfgMain::BM) forced_row_tile = rows;
+  return before;
 }
 
 extern "C" int64_t moe_dgate_blocks(int64_t I) {
@@ -1119,14 +1158,16 @@ static int dgrad_down_impl(const uint16_t* dyp, const uint16_t* w2, const uint16
   if (R == 0) return 0;
   MOE_CHECK_PTR(dyp); MOE_CHECK_PTR(w2); MOE_CHECK_PTR(g); MOE_CHECK_PTR(u);
   MOE_CHECK_PTR(dg); MOE_CHECK_PTR(du);
-  using Cfg = CfgMain;
-  GemmArgs a{};
-  a.C2 = dgate_part;
-  a.A0 = dyp; a.B0 = w2; a.X0 = g; a.X1 = u; a.C0 = dg; a.C1 = du; a.offs = offs;
-  a.E = (int)E; a.R = (int)R; a.N = (int)I; a.K = (int)H; a.ld_c = (int)ld_out;
-  a.n_tiles = (int)((I + Cfg::BN - 1) / Cfg::BN);
-  a.m_slots = row_slots<Cfg>(R, E);
-  return launch<DGRAD_DOWN, Cfg, uint16_t>(a, (long long)a.n_tiles * a.m_slots, (hipStream_t)stream);
+  return with_row_tile(small_row_tiles(R, E, I), [&](auto cfg) {
+    using Cfg = decltype(cfg);
+    GemmArgs a{};
+    a.C2 = dgate_part;
+    a.A0 = dyp; a.B0 = w2; a.X0 = g; a.X1 = u; a.C0 = dg; a.C1 = du; a.offs = offs;
+    a.E = (int)E; a.R = (int)R; a.N = (int)I; a.K = (int)H; a.ld_c = (int)ld_out;
+    a.n_tiles = (int)((I + Cfg::BN - 1) / Cfg::BN);
+    a.m_slots = row_slots<Cfg>(R, E);
+    return launch<DGRAD_DOWN, Cfg, uint16_t>(a, (long long)a.n_tiles * a.m_slots, (hipStream_t)stream);
+  });
 }
 
 extern "C" int moe_gemm_dgrad_down_swiglu_bwd(const uint16_t* dyp, const uint16_t* w2,
@@ -1154,14 +1195,16 @@ extern "C" int moe_gemm_dgrad_down_swiglu_bwd_blocked(const uint16_t* dyp, const
   if (R == 0) return 0;
   MOE_CHECK_PTR(dyp); MOE_CHECK_PTR(w2); MOE_CHECK_PTR(gu_blocked); MOE_CHECK_PTR(dg); MOE_CHECK_PTR(du);
   if (ld_out != 0 && (ld_out < I || (ld_out % 8) != 0 || ld_out > (1 << 17))) return MOE_ERR_SHAPE;
-  using Cfg = CfgMain;
-  GemmArgs a{};
-  a.C2 = dgate_part;
-  a.A0 = dyp; a.B0 = w2; a.X0 = (const uint16_t*)gu_blocked; a.C0 = dg; a.C1 = du; a.offs = offs;
-  a.E = (int)E; a.R = (int)R; a.N = (int)I; a.K = (int)H; a.ld_c = (int)ld_out;
-  a.n_tiles = (int)((I + Cfg::BN - 1) / Cfg::BN);
-  a.m_slots = row_slots<Cfg>(R, E);
-  return launch<DGRAD_DOWN, Cfg, uint16_t, true>(a, (long long)a.n_tiles * a.m_slots, (hipStream_t)stream);
+  return with_row_tile(small_row_tiles(R, E, I), [&](auto cfg) {
+    using Cfg = decltype(cfg);
+    GemmArgs a{};
+    a.C2 = dgate_part;
+    a.A0 = dyp; a.B0 = w2; a.X0 = (const uint16_t*)gu_blocked; a.C0 = dg; a.C1 = du; a.offs = offs;
+    a.E = (int)E; a.R = (int)R; a.N = (int)I; a.K = (int)H; a.ld_c = (int)ld_out;
+    a.n_tiles = (int)((I + Cfg::BN - 1) / Cfg::BN);
+    a.m_slots = row_slots<Cfg>(R, E);
+    return launch<DGRAD_DOWN, Cfg, uint16_t, true>(a, (long long)a.n_tiles * a.m_slots, (hipStream_t)stream);
+  });
 }
 
 // The two row gradients side by side in one buffer: dgu [R, 2I], row = [dg row | du row].  The
@@ -1182,13 +1225,15 @@ static int dgrad_gateup_impl(const uint16_t* dg, const uint16_t* du, int64_t ld_
   if (int rc = check_common(offs, E, R, H, I)) return rc;
   if (R == 0) return 0;
   MOE_CHECK_PTR(dg); MOE_CHECK_PTR(du); MOE_CHECK_PTR(w1); MOE_CHECK_PTR(w3); MOE_CHECK_PTR(dxp);
-  using Cfg = CfgMain;
-  GemmArgs a{};
-  a.A0 = dg; a.A1 = du; a.B0 = w1; a.B1 = w3; a.C0 = dxp; a.offs = offs; a.ld_a = (int)ld_in;
-  a.E = (int)E; a.R = (int)R; a.N = (int)H; a.K = (int)I;
-  a.n_tiles = (int)((H + Cfg::BN - 1) / Cfg::BN);
-  a.m_slots = row_slots<Cfg>(R, E);
-  return launch<DGRAD_GATEUP, Cfg, uint16_t>(a, (long long)a.n_tiles * a.m_slots, (hipStream_t)stream);
+  return with_row_tile(small_row_tiles(R, E, H), [&](auto cfg) {
+    using Cfg = decltype(cfg);
+    GemmArgs a{};
+    a.A0 = dg; a.A1 = du; a.B0 = w1; a.B1 = w3; a.C0 = dxp; a.offs = offs; a.ld_a = (int)ld_in;
+    a.E = (int)E; a.R = (int)R; a.N = (int)H; a.K = (int)I;
+    a.n_tiles = (int)((H + Cfg::BN - 1) / Cfg::BN);
+    a.m_slots = row_slots<Cfg>(R, E);
+    return launch<DGRAD_GATEUP, Cfg, uint16_t>(a, (long long)a.n_tiles * a.m_slots, (hipStream_t)stream);
+  });
 }
 
 extern "C" int moe_gemm_dgrad_gateup_packed(const uint16_t* dgu, const uint16_t* w1, const uint16_t* w3,

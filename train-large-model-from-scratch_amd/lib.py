@@ -29,6 +29,7 @@ SIGNATURES = {
     "moe_gemm_gateup_swiglu_fwd_blocked": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _vp]),
     "moe_gemm_dgrad_down_swiglu_bwd_blocked": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _i64,
                                                       _vp, _vp]),
+    "moe_gemm_force_row_tile": (_int, [_int]),
     "moe_gemm_down_fwd": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp]),
     "moe_gemm_dgrad_down_swiglu_bwd": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _vp]),
     "moe_dgate_blocks": (_i64, [_i64]),
