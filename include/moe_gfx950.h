@@ -237,6 +237,21 @@ int moe_gemm_wgrad_pair(const uint16_t* dgu, const uint16_t* xp, const int32_t* 
  * partial sums per expert, to be added in a fixed order.  E*S <= 1024.  (No counterpart in
  * the reference, whose bmm does not split the contraction.) */
 int moe_segment_offsets(const int32_t* offs, int64_t E, int64_t S, int32_t* seg, void* stream);
+/* The same idea with segments of bounded length, for skewed routing: expert e is cut into
+ * ceil(n_e / L) equal parts, so that an expert with 40 % of the rows gets 40 % of the segments and
+ * the longest contraction of the launch is L rows whatever the routing.  Segments are numbered
+ * expert by expert: seg_start int32 [E+1] (seg_start[e] = e's first segment, seg_start[E] = how many
+ * are used), seg int32 [S_max+1] with S_max = moe_segments_by_length_max(R, E, L) = ceil(R/L) + E
+ * (a bound that holds for every routing; the slots past the used ones are empty segments at the end
+ * of the rows).  moe_gemm_wgrad over seg with S_max "experts" and fp32 output gives the partial
+ * sums; moe_wgrad_reduce_segments adds each expert's partials in ascending order (reproducible)
+ * into dw [E,M,N] of dw_dtype: dw[e] (+)= sum_s part[s], exact zeros for experts without rows
+ * (left untouched when accumulate != 0).  S_max <= 1024.  (No counterpart in the reference.) */
+int64_t moe_segments_by_length_max(int64_t R, int64_t E, int64_t L);
+int moe_segment_offsets_by_length(const int32_t* offs, int64_t E, int64_t L, int64_t S_max,
+                                  int32_t* seg, int32_t* seg_start, void* stream);
+int moe_wgrad_reduce_segments(const float* part, const int32_t* seg_start, int64_t E, int64_t M,
+                              int64_t N, void* dw, int dw_dtype, int accumulate, void* stream);
 
 /* ---- combine ------------------------------------------------------------------------
  * Replaces the un-sorts, the gate scaling and the sum over k (mlp.py:160-167):

@@ -457,6 +457,30 @@ def test_expert_gemms_forward_backward(ops, R, H, I, E, empty):
         assert torch.allclose(part, again, rtol=1e-4, atol=1e-4 * float(again.abs().max()))
         for e in empty:
             assert not part[e].any()
+    # segments of bounded length (what the autograd functions use): exact bounds against numpy,
+    # the fixed-order reduction against the unsplit product, fresh and accumulating, both dtypes
+    for Lseg in (64, 200, 4096):
+        seg, seg_start, S_max = ops.segment_offsets_by_length(offs, E, Lseg, R)
+        o = offs.cpu().numpy().astype(np.int64)
+        n = o[1:] - o[:-1]
+        ns = -(-n // Lseg)
+        assert S_max == -(-R // Lseg) + E and ns.sum() <= S_max
+        assert seg_start.cpu().tolist() == [0] + np.cumsum(ns).tolist()
+        want = [int(o[e] + n[e] * j // ns[e]) for e in range(E) for j in range(ns[e])]
+        want += [int(o[E])] * (S_max + 1 - len(want))
+        assert seg.cpu().tolist() == want
+        if S_max > 1024:
+            continue
+        part = ops.gemm_wgrad(dyp.cuda(), act, seg, S_max, torch.float32)
+        red = ops.wgrad_reduce_segments(part, seg_start, E, torch.float32)
+        assert torch.allclose(red, again, rtol=1e-4, atol=1e-4 * float(again.abs().max()))
+        assert torch.equal(red, ops.wgrad_reduce_segments(part, seg_start, E, torch.float32))
+        for e in empty:
+            assert not red[e].any()
+        red16 = ops.wgrad_reduce_segments(part, seg_start, E, torch.bfloat16)
+        assert torch.equal(red16, red.to(torch.bfloat16))
+        acc2 = ops.wgrad_reduce_segments(part, seg_start, E, torch.float32, out=base.clone().cuda())
+        assert torch.allclose(acc2, red + base.cuda(), rtol=1e-6, atol=1e-6)
 
 
 @pytest.mark.parametrize("R,H,I,E,empty", [(1000, 256, 128, 5, ()), (777, 200, 72, 7, (2, 5)),

@@ -803,6 +803,102 @@ extern "C" int moe_segment_offsets(const int32_t* offs, int64_t E, int64_t S, in
   return moe_launch_status();
 }
 
+// Row segments of at most L rows each: expert e is cut into ceil(n_e / L) equal parts, numbered
+// expert by expert.  seg_start[e] = index of e's first segment (seg_start[E] = their number);
+// seg[s] = first row of segment s; the slots past the last used one, up to S_max, are empty
+// segments at the end of the rows.  One wave: a scan over the experts' segment counts.
+__global__ void segments_by_length_kernel(const int32_t* __restrict__ offs, int E, int L, int S_max,
+                                          int32_t* __restrict__ seg, int32_t* __restrict__ seg_start) {
+  const int lane = threadIdx.x;
+  int carry = 0;
+  for (int b = 0; b < E; b += MOE_WAVE) {
+    const int e = b + lane;
+    const int lo = e < E ? offs[e] : 0;
+    const int n = e < E ? offs[e + 1] - lo : 0;
+    const int ns = (n + L - 1) / L;
+    int incl = ns;
+#pragma unroll
+    for (int off = 1; off < MOE_WAVE; off <<= 1) {
+      const int o = __shfl_up(incl, off, MOE_WAVE);
+      if (lane >= off) incl += o;
+    }
+    const int start = carry + incl - ns;
+    if (e < E) {
+      seg_start[e] = start;
+      for (int j = 0; j < ns; ++j) seg[start + j] = lo + (int32_t)((long long)n * j / ns);
+    }
+    carry += __shfl(incl, MOE_WAVE - 1, MOE_WAVE);
+  }
+  if (lane == 0) seg_start[E] = carry;
+  const int R = offs[E];
+  for (int s2 = carry + lane; s2 <= S_max; s2 += MOE_WAVE) seg[s2] = R;
+}
+
+extern "C" int64_t moe_segments_by_length_max(int64_t R, int64_t E, int64_t L) {
+  if (R < 0 || E <= 0 || L <= 0) return 0;
+  return (R + L - 1) / L + E;
+}
+
+extern "C" int moe_segment_offsets_by_length(const int32_t* offs, int64_t E, int64_t L, int64_t S_max,
+                                             int32_t* seg, int32_t* seg_start, void* stream) {
+  if (!offs || !seg || !seg_start) return MOE_ERR_NULL;
+  if (E <= 0 || L <= 0 || S_max < E) return MOE_ERR_SHAPE;
+  if (E > 1024 || S_max > 1024 || L > (int64_t)1 << 30) return MOE_ERR_LIMIT;
+  hipLaunchKernelGGL(segments_by_length_kernel, dim3(1), dim3(MOE_WAVE), 0, (hipStream_t)stream, offs,
+                     (int)E, (int)L, (int)S_max, seg, seg_start);
+  return moe_launch_status();
+}
+
+// dw[e] (+)= sum of part[s] over e's segments in ascending order; 8 elements per thread.
+template <typename OutT>
+__global__ void reduce_segments_kernel(const float* __restrict__ part, const int32_t* __restrict__ seg_start,
+                                       int E, long long mn8, OutT* __restrict__ dw, int accumulate) {
+  const long long total = (long long)E * mn8;
+  for (long long idx = blockIdx.x * (long long)blockDim.x + threadIdx.x; idx < total;
+       idx += (long long)gridDim.x * blockDim.x) {
+    const int e = (int)(idx / mn8);
+    const long long i = idx - (long long)e * mn8;
+    const int s0 = seg_start[e], s1 = seg_start[e + 1];
+    Row8 acc;
+#pragma unroll
+    for (int v = 0; v < 8; ++v) acc.v[v] = 0.f;
+    for (int sg = s0; sg < s1; ++sg) {
+      const Row8 r = load8(part + ((long long)sg * mn8 + i) * 8);
+#pragma unroll
+      for (int v = 0; v < 8; ++v) acc.v[v] += r.v[v];
+    }
+    OutT* dst = dw + idx * 8;
+    if (accumulate) {
+      const Row8 old = load8(dst);
+#pragma unroll
+      for (int v = 0; v < 8; ++v) acc.v[v] += old.v[v];
+    }
+    store8(dst, acc);
+  }
+}
+
+extern "C" int moe_wgrad_reduce_segments(const float* part, const int32_t* seg_start, int64_t E, int64_t M,
+                                         int64_t N, void* dw, int dw_dtype, int accumulate, void* stream) {
+  if (!seg_start) return MOE_ERR_NULL;
+  if (E <= 0 || M <= 0 || N <= 0 || (M % 8) || (N % 8)) return MOE_ERR_SHAPE;
+  if (E > 1024 || M > (1 << 16) || N > (1 << 16)) return MOE_ERR_LIMIT;
+  MOE_CHECK_PTR(part);
+  MOE_CHECK_PTR(dw);
+  const long long mn8 = M * N / 8;
+  long long blocks = (E * mn8 + 255) / 256;
+  if (blocks > 256 * 8) blocks = 256 * 8;
+  hipStream_t st = (hipStream_t)stream;
+  if (dw_dtype == MOE_DT_F32)
+    hipLaunchKernelGGL(reduce_segments_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, st, part, seg_start,
+                       (int)E, mn8, (float*)dw, accumulate);
+  else if (dw_dtype == MOE_DT_BF16)
+    hipLaunchKernelGGL(reduce_segments_kernel<uint16_t>, dim3((unsigned)blocks), dim3(256), 0, st, part, seg_start,
+                       (int)E, mn8, (uint16_t*)dw, accumulate);
+  else
+    return MOE_ERR_DTYPE;
+  return moe_launch_status();
+}
+
 extern "C" int moe_cast_f32_bf16(const float* src, uint16_t* dst, int64_t n, void* stream) {
   if (n == 0) return 0;
   MOE_CHECK_PTR(src);

@@ -108,34 +108,47 @@ def _compute_units(device) -> int:
 
 
 def _wgrad_split(E: int, M: int, N: int, device) -> int:
-    """Into how many row segments each expert's contraction is cut.  The weight-gradient
-    kernel makes one workgroup per 256 x 256 output tile and expert; with few experts and
-    small matrices that is a fraction of the chip, and under skewed routing the one tile row
-    of the largest expert sets the time.  Cutting every expert's rows into S segments gives
-    S times the tiles, each 1/S as long (decided from shapes alone: no look at the counts,
-    no host synchronisation)."""
+    """Whether (> 1) the weight-gradient launch for [E, M, N] is too small to fill the chip: the
+    kernel makes one workgroup per 256 x 256 output tile and expert; with few experts and small
+    matrices that is a fraction of the compute units, and under skewed routing the tiles of the
+    largest expert set the time.  Decided from shapes alone (no look at the counts, no host
+    synchronisation)."""
     tiles = E * -(-M // _WGRAD_TILE) * -(-N // _WGRAD_TILE)
-    return max(1, min(8, _compute_units(device) // max(tiles, 1), 1024 // max(E, 1)))
+    return max(1, _compute_units(device) // max(tiles, 1))
+
+
+def _segment_rows(E: int, M: int, N: int, R: int, device) -> int:
+    """Row segment length L for a small launch: every expert's contraction is cut into
+    ceil(n_e / L) equal parts, so that the (ceil(R/L) + E) x tiles jobs about fill the compute
+    units once and none contracts over more than L rows, however skewed the routing."""
+    tiles = -(-M // _WGRAD_TILE) * -(-N // _WGRAD_TILE)   # per expert
+    free = max(_compute_units(device) - E * tiles, tiles)
+    L = -(-R * tiles // free)
+    L = max(256, -(-L // 64) * 64)
+    while -(-R // L) + E > 1024:   # the launch takes at most 1024 segments
+        L *= 2
+    return L
 
 
 def _gemm_wgrad(a, b, offs, E, dtype, out=None, segs=None):
-    """dw[e] (+)= a[rows of e]^T b[rows of e], cut along the rows when that fills the chip
-    better: the segments are the "experts" of one launch with fp32 results, summed in a fixed
-    order (reproducible).  `segs` (a dict that lives as long as one backward pass) keeps the
-    segment bounds of these `offs` per split, so that the three stacks share them."""
-    M, N = a.shape[1], b.shape[1]
-    S = _wgrad_split(E, M, N, a.device)
-    if S == 1 or a.shape[0] == 0:
+    """dw[e] (+)= a[rows of e]^T b[rows of e], cut along the rows when the launch would otherwise
+    leave most of the chip idle: the segments are the "experts" of one launch with fp32 results,
+    which a second kernel adds per expert in a fixed order (reproducible).  `segs` (a dict that
+    lives as long as one backward pass) keeps the segments of these `offs` per length, so that the
+    three stacks share them."""
+    R, M = a.shape
+    N = b.shape[1]
+    if R == 0 or _wgrad_split(E, M, N, a.device) < 2:
         return ops.gemm_wgrad(a, b, offs, E, dtype, out=out)
-    seg_offs = None if segs is None else segs.get(S)
-    if seg_offs is None:
-        seg_offs = ops.segment_offsets(offs, E, S)
+    L = _segment_rows(E, M, N, R, a.device)
+    held = None if segs is None else segs.get(L)
+    if held is None:
+        held = ops.segment_offsets_by_length(offs, E, L, R)
         if segs is not None:
-            segs[S] = seg_offs
-    part = ops.gemm_wgrad(a, b, seg_offs, E * S, torch.float32).view(E, S, M, N).sum(1)
-    if out is None:
-        return part.to(dtype)
-    return out.add_(part)
+            segs[L] = held
+    seg, seg_start, S_max = held
+    part = ops.gemm_wgrad(a, b, seg, S_max, torch.float32)
+    return ops.wgrad_reduce_segments(part, seg_start, E, dtype, out=out)
 
 
 def _wgrad(a, b, offs, E, wdtype, needed, param, segs=None):
@@ -167,7 +180,7 @@ def _pair_ok(E, I, H, need_w, into, device):
     [dg | du] buffer: both wanted, 256-row tiles of the stacked result do not straddle the halves,
     the launch fills the chip without a row split, and (when the kernel is to add into `.grad`)
     both slots are in the same state."""
-    if not (need_w[0] and need_w[1]) or I % _WGRAD_TILE != 0 or _wgrad_split(E, I, H, device) != 1:
+    if not (need_w[0] and need_w[1]) or I % _WGRAD_TILE != 0 or _wgrad_split(E, I, H, device) >= 2:
         return False
     p1, p3 = into[0], into[1]
     if p1 is None and p3 is None:

@@ -43,6 +43,9 @@ SIGNATURES = {
     "moe_gemm_dgrad_gateup_packed": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp]),
     "moe_gemm_wgrad_pair": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _int, _int, _vp]),
     "moe_segment_offsets": (_int, [_vp, _i64, _i64, _vp, _vp]),
+    "moe_segments_by_length_max": (_i64, [_i64, _i64, _i64]),
+    "moe_segment_offsets_by_length": (_int, [_vp, _i64, _i64, _i64, _vp, _vp, _vp]),
+    "moe_wgrad_reduce_segments": (_int, [_vp, _vp, _i64, _i64, _i64, _vp, _int, _int, _vp]),
     "moe_combine_fwd": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp, _int, _vp]),
     "moe_combine_bwd": (_int, [_vp, _int, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _vp]),
     "moe_combine_fwd_residual": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _int, _vp]),

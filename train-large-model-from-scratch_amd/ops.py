@@ -266,6 +266,31 @@ def segment_offsets(offs: torch.Tensor, E: int, S: int) -> torch.Tensor:
     return seg
 
 
+def segment_offsets_by_length(offs: torch.Tensor, E: int, L: int, R: int):
+    """offs int32 [E+1] -> (seg int32 [S_max+1], seg_start int32 [E+1], S_max): every expert's rows cut
+    into ceil(n_e / L) equal parts, numbered expert by expert; S_max = ceil(R/L) + E bounds their
+    number for any routing (unused slots are empty segments)."""
+    L_ = _lib.load()
+    S_max = int(L_.cdll.moe_segments_by_length_max(R, E, L))
+    seg = torch.empty(S_max + 1, dtype=torch.int32, device=offs.device)
+    seg_start = torch.empty(E + 1, dtype=torch.int32, device=offs.device)
+    L_.call("moe_segment_offsets_by_length", _p(offs), E, L, S_max, _p(seg), _p(seg_start), _stream())
+    return seg, seg_start, S_max
+
+
+def wgrad_reduce_segments(part: torch.Tensor, seg_start: torch.Tensor, E: int, dtype: torch.dtype,
+                          out: torch.Tensor | None = None):
+    """part fp32 [S_max, M, N] -> dw [E, M, N]: each expert's partial sums added in ascending order;
+    `out` accumulates."""
+    _, M, N = part.shape
+    acc = out is not None
+    if out is None:
+        out = torch.empty(E, M, N, dtype=dtype, device=part.device)
+    _lib.load().call("moe_wgrad_reduce_segments", _p(part), _p(seg_start), E, M, N, _p(out), _dt(out),
+                     1 if acc else 0, _stream())
+    return out
+
+
 def combine_fwd(y, gates, row_to_pos, T: int, k: int, dtype: torch.dtype):
     H = y.shape[-1]
     out = torch.empty(T, H, dtype=dtype, device=y.device)
