@@ -149,6 +149,108 @@ __global__ __launch_bounds__(256) void positions_kernel(const int32_t* __restric
   }
 }
 
+// The three kernels above as one, for inputs small enough that a single workgroup's LDS holds
+// every chunk's histogram (SMALL_MAX_CHUNKS * E ints): 16 waves take the 256-row chunks in turn,
+// the histograms, their column scans and the running cursors never leave LDS, and two launches
+// (and their gaps) are saved where the whole layer step is a few tens of microseconds.  Same
+// chunking, same stable ranks: the results are the same bits as the three-kernel path.
+constexpr int SMALL_WAVES = 16;
+constexpr int SMALL_MAX_CHUNKS = 64;         // R <= 16384
+constexpr int SMALL_MAX_WORDS = 12 * 1024;   // chunks * E ints of LDS (48 KB)
+
+__global__ __launch_bounds__(SMALL_WAVES* MOE_WAVE) void dispatch_small_kernel(
+    const int32_t* __restrict__ ids, int R, int E, int NW, int32_t* __restrict__ counts,
+    int32_t* __restrict__ offs, int32_t* __restrict__ pos_to_row, int32_t* __restrict__ row_to_pos,
+    int32_t* __restrict__ bad_total) {
+  extern __shared__ int sm[];  // [NW][E] chunk histograms, later write cursors; [E] starts; [1] bad
+  int* whist = sm;
+  int* starts = sm + NW * E;
+  int* bad_sum = starts + E;
+  const int lane = lane_id(), wv = threadIdx.x / MOE_WAVE;
+  for (int i = threadIdx.x; i < NW * E + E + 1; i += blockDim.x) sm[i] = 0;
+  __syncthreads();
+  // per-chunk histograms
+  int bad = 0;
+  for (int w = wv; w < NW; w += SMALL_WAVES) {
+    const int base = w * ROWS_PER_WAVE;
+#pragma unroll
+    for (int it = 0; it < ROWS_PER_WAVE / MOE_WAVE; ++it) {
+      const int r = base + it * MOE_WAVE + lane;
+      if (r < R) {
+        const int e = ids[r];
+        bad += (e < 0 || e >= E) ? 1 : 0;
+        atomicAdd(&whist[w * E + clamp_expert(e, E)], 1);
+      }
+    }
+  }
+#pragma unroll
+  for (int off = MOE_WAVE / 2; off > 0; off >>= 1) bad += __shfl_xor(bad, off, MOE_WAVE);
+  if (lane == 0 && bad) atomicAdd(bad_sum, bad);
+  __syncthreads();
+  // exclusive scan down every expert's column of chunk counts (NW <= 64: one pass of a wave)
+  for (int e = wv; e < E; e += SMALL_WAVES) {
+    const int v = lane < NW ? whist[lane * E + e] : 0;
+    const int incl = wave_incl_scan(v);
+    if (lane < NW) whist[lane * E + e] = incl - v;
+    if (lane == MOE_WAVE - 1) {
+      starts[e] = incl;  // the expert's count, for the moment
+      counts[e] = incl;
+    }
+  }
+  __syncthreads();
+  // exclusive scan of the counts over the experts (wave 0), then the cursors of every chunk
+  if (wv == 0) {
+    int carry = 0;
+    for (int b = 0; b < E; b += MOE_WAVE) {
+      const int e = b + lane;
+      const int c = e < E ? starts[e] : 0;
+      const int incl = wave_incl_scan(c);
+      if (e < E) {
+        const int st = carry + incl - c;
+        starts[e] = st;
+        offs[e] = st;
+      }
+      carry += __shfl(incl, MOE_WAVE - 1, MOE_WAVE);  // (every lane takes part: not inside the branch)
+    }
+    if (lane == 0) {
+      offs[E] = carry;
+      if (bad_total) *bad_total = *bad_sum;
+    }
+  }
+  __syncthreads();
+  int nbits = 0;
+  while ((1 << nbits) < E) ++nbits;
+  for (int w = wv; w < NW; w += SMALL_WAVES) {
+    int* cur = whist + w * E;
+    for (int e = lane; e < E; e += MOE_WAVE) cur[e] += starts[e];
+    __builtin_amdgcn_wave_barrier();
+    const int base = w * ROWS_PER_WAVE;
+    for (int it = 0; it < ROWS_PER_WAVE / MOE_WAVE; ++it) {
+      const int r = base + it * MOE_WAVE + lane;
+      const bool valid = r < R;
+      const int e = valid ? clamp_expert(ids[r], E) : 0;
+      unsigned long long mask = __ballot(valid);
+      for (int b = 0; b < nbits; ++b) {
+        const bool bit = (e >> b) & 1;
+        const unsigned long long bal = __ballot(valid && bit);
+        mask &= bit ? bal : ~bal;
+      }
+      const unsigned long long lt = (1ull << lane) - 1ull;
+      const int rank = __popcll(mask & lt);
+      int old = 0;
+      if (valid) old = cur[e];
+      __builtin_amdgcn_wave_barrier();
+      if (valid && rank == 0) cur[e] = old + __popcll(mask);
+      __builtin_amdgcn_wave_barrier();
+      if (valid) {
+        const int pos = old + rank;
+        pos_to_row[pos] = r;
+        row_to_pos[r] = pos;
+      }
+    }
+  }
+}
+
 // ---- row movers ---------------------------------------------------------------------------
 
 constexpr int ROWS_PER_BLOCK = 4;
@@ -458,6 +560,12 @@ int histogram_scan_impl(const int32_t* ids, int64_t R, int64_t E, int32_t* count
                         int32_t* pos_to_row, int32_t* row_to_pos, int32_t* bad_ids, void* scratch,
                         hipStream_t s) {
   const int NW = (int)((R + ROWS_PER_WAVE - 1) / ROWS_PER_WAVE);
+  if (NW > 0 && NW <= SMALL_MAX_CHUNKS && (int64_t)NW * E <= SMALL_MAX_WORDS) {
+    const size_t lds_small = ((size_t)NW * E + E + 1) * sizeof(int);
+    hipLaunchKernelGGL(dispatch_small_kernel, dim3(1), dim3(SMALL_WAVES * MOE_WAVE), lds_small, s, ids, (int)R,
+                       (int)E, NW, counts, offs, pos_to_row, row_to_pos, bad_ids);
+    return moe_launch_status();
+  }
   const int nblk = NW > 0 ? (NW + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK : 1;
   const size_t lds = (size_t)WAVES_PER_BLOCK * E * sizeof(int);
   int32_t* whist = (int32_t*)scratch;
