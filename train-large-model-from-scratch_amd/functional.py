@@ -108,11 +108,11 @@ def _compute_units(device) -> int:
 
 
 def _wgrad_split(E: int, M: int, N: int, device) -> int:
-    """Whether (> 1) the weight-gradient launch for [E, M, N] is too small to fill the chip: the
-    kernel makes one workgroup per 256 x 256 output tile and expert; with few experts and small
-    matrices that is a fraction of the compute units, and under skewed routing the tiles of the
-    largest expert set the time.  Decided from shapes alone (no look at the counts, no host
-    synchronisation)."""
+    """Compute units per output tile of the weight-gradient launch for [E, M, N] (at least 1).
+    The kernel makes one workgroup per 256 x 256 output tile and expert; with few experts and
+    small matrices that is a fraction of the chip, and under skewed routing the tiles of the
+    largest expert set the time: from 2 on, the contraction is cut into row segments.  Decided
+    from shapes alone (no look at the counts, no host synchronisation)."""
     tiles = E * -(-M // _WGRAD_TILE) * -(-N // _WGRAD_TILE)
     return max(1, _compute_units(device) // max(tiles, 1))
 
