@@ -28,18 +28,17 @@ HBM_PEAK_GBS = 8000.0
 # are in profiles/grouped_gemm_cfg3_pmc.txt.  bench.py cannot run the profiler on itself, so
 # the figures are carried here and refreshed whenever that profile is.
 MEASURED_HBM_BYTES_PER_LAUNCH = {
-    (3, "gemm_gateup_swiglu_fwd"): 4.009e9,
-    (3, "gemm_down_fwd"): 1.829e9,
-    (3, "gemm_dgrad_down_swiglu_bwd"): 2.465e9,
-    (3, "gemm_dgrad_gateup"): 3.771e9,
+    (3, "gemm_gateup_swiglu_fwd_blocked"): 4.019e9,
+    (3, "gemm_gateup_swiglu_fwd"): 4.019e9,
+    (3, "gemm_down_fwd"): 1.849e9,
+    (3, "gemm_dgrad_down_swiglu_bwd_blocked"): 2.452e9,
+    (3, "gemm_dgrad_down_swiglu_bwd"): 2.452e9,
+    (3, "gemm_dgrad_gateup_packed"): 3.760e9,
+    (3, "gemm_dgrad_gateup"): 3.760e9,
     (3, "gemm_wgrad_down"): 1.074e9,
-    (3, "gemm_wgrad_gate_and_up_pair"): 2.23e9,   # from the average over both weight-gradient launches
-    # the same kernels under the names of their entry points (as the in-step events see them)
-    (3, "gemm_dgrad_down_swiglu_bwd_packed"): 2.465e9,
-    (3, "gemm_dgrad_gateup_packed"): 3.771e9,
-    (3, "gemm_wgrad_pair"): 2.23e9,
-    (3, "gemm_gateup_swiglu_fwd_blocked"): 4.009e9,
-    (3, "gemm_dgrad_down_swiglu_bwd_blocked"): 2.465e9,
+    (3, "gemm_wgrad"): 1.074e9,
+    (3, "gemm_wgrad_pair"): 2.18e9,                # from the average over both weight-gradient launches
+    (3, "gemm_wgrad_gate_and_up_pair"): 2.18e9,
 }
 
 
