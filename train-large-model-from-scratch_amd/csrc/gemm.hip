@@ -721,10 +721,11 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WAVES_PER_SIMD) void grouped_gemm_ker
       b.g[j][0] = b.g[j][1] = b.u[j][0] = b.u[j][1] = zero;
       if (t.row0 + wm * WTM + i * 32 < t.row_end && cb < n_cb) {
         const u32x4* rec = reinterpret_cast<const u32x4*>(gu_block(p.X0, t, wm * FM + i, cb, lane_e));
-        b.g[j][0] = rec[0];
-        b.g[j][1] = rec[64];
-        b.u[j][0] = rec[128];
-        b.u[j][1] = rec[192];
+        // (read exactly once: streamed past the L2 lines the operand panels live in)
+        b.g[j][0] = __builtin_nontemporal_load(rec + 0);
+        b.g[j][1] = __builtin_nontemporal_load(rec + 64);
+        b.u[j][0] = __builtin_nontemporal_load(rec + 128);
+        b.u[j][1] = __builtin_nontemporal_load(rec + 192);
       }
     };
     RowRegs rows_in;
@@ -760,8 +761,10 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WAVES_PER_SIMD) void grouped_gemm_ker
                 const int cb = (col_w0 + j * 32) / 32;
                 if (p.C0 && strip_live && cb < n_cb) {
                   u32x4* rec = reinterpret_cast<u32x4*>(gu_block(p.C0, t, wm * FM + i, cb, lane_e));
-                  rec[64 * (q >> 1)] = u32x4{gq[0][0], gq[0][1], gq[1][0], gq[1][1]};
-                  rec[128 + 64 * (q >> 1)] = u32x4{uq[0][0], uq[0][1], uq[1][0], uq[1][1]};
+                  // (written once, read by the backward pass much later: streaming stores)
+                  __builtin_nontemporal_store(u32x4{gq[0][0], gq[0][1], gq[1][0], gq[1][1]}, rec + 64 * (q >> 1));
+                  __builtin_nontemporal_store(u32x4{uq[0][0], uq[0][1], uq[1][0], uq[1][1]},
+                                              rec + 128 + 64 * (q >> 1));
                 }
               }
             } else if (p.C0) {
