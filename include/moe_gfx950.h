@@ -318,6 +318,43 @@ int moe_rmsnorm_bwd(const void* x, int x_dtype, const float* weight, const float
  * mlp.py:154-157 under trainer.py:209-211). */
 int moe_cast_f32_bf16(const float* src, uint16_t* dst, int64_t n, void* stream);
 
+/* ---- the path in fp32 ---------------------------------------------------------------
+ * For a layer that runs without autocast on fp32 tensors: the reference then keeps every
+ * step of mlp.py:104-169 in fp32 (the three bmm's of :154-157 included) and so do these
+ * entry points.  Routing and dispatch are the entries above (fp32 logits).  Expert-contiguous
+ * buffers are fp32 here: xp, dyp, dxp, y [R,H]; g, u, act, dact, dg, du [R,I].  H and I must be
+ * multiples of 4 (16-byte accesses); weights are the fp32 parameters themselves. */
+
+/* mlp.py:104-131 (repeat_interleave + both sorts): xp[pos,:] = x[pos_to_row[pos] / k, :]. */
+int moe_f32_gather_rows(const float* x, const int32_t* pos_to_row, int64_t T, int64_t R, int64_t H,
+                        int64_t k, float* xp, void* stream);
+/* mlp.py:160-169: out[t,:] = sum_j gates[t*k+j] * y[row_to_pos[t*k+j],:], j ascending. */
+int moe_f32_combine_fwd(const float* y, const float* gates, const int32_t* row_to_pos, int64_t T,
+                        int64_t H, int64_t k, float* out, void* stream);
+/* Its backward: dyp[pos,:] = gates[row] * dy[row / k,:] and, unless dgates is NULL,
+ * dgates[row] = <dy[row / k,:], y[pos,:]> (row = pos_to_row[pos]; y may be NULL with dgates). */
+int moe_f32_combine_bwd(const float* dy, const float* y, const float* gates, const int32_t* pos_to_row,
+                        int64_t T, int64_t R, int64_t H, int64_t k, float* dyp, float* dgates,
+                        void* stream);
+/* Backward of the gather: dx[t,:] = sum_j dxp[row_to_pos[t*k+j],:], j ascending. */
+int moe_f32_permute_bwd(const float* dxp, const int32_t* row_to_pos, int64_t T, int64_t H, int64_t k,
+                        float* dx, void* stream);
+/* mlp.py:156: act = silu(g) * u over n elements (n a multiple of 4), and its backward
+ * dg = dact * u * silu'(g), du = dact * silu(g). */
+int moe_f32_swiglu_fwd(const float* g, const float* u, int64_t n, float* act, void* stream);
+int moe_f32_swiglu_bwd(const float* dact, const float* g, const float* u, int64_t n, float* dg,
+                       float* du, void* stream);
+/* The bmm's of mlp.py:154-157 and their input gradients over ragged expert rows (no padding):
+ * c[r,:] (+)= a[r,:] x B_e for the rows r of expert e; a [R,K], c [R,N], b [E,N,K] when
+ * b_k_contiguous (c = a b_e^T: x W1^T, x W3^T, act W2^T) or [E,K,N] otherwise (c = a b_e:
+ * dy W2, dg W1, du W3).  accumulate != 0 adds into c. */
+int moe_f32_gemm_rows(const float* a, const float* b, const int32_t* offs, int64_t E, int64_t R,
+                      int64_t N, int64_t K, int b_k_contiguous, float* c, int accumulate, void* stream);
+/* Their weight gradients: dw[e] (+)= a[rows of e]^T b[rows of e]; a [R,M], b [R,N], dw [E,M,N].
+ * Experts without rows get exact zeros (are left untouched when accumulating). */
+int moe_f32_gemm_wgrad(const float* a, const float* b, const int32_t* offs, int64_t E, int64_t R,
+                       int64_t M, int64_t N, float* dw, int accumulate, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

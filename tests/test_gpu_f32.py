@@ -1,0 +1,257 @@
+"""GPU parity tests of the fp32 path (the layer called without autocast on fp32 tensors, where the
+reference computes every step of model/modules/mlp.py:101-169 in fp32).  Called through the C ABI
+and checked against fp64 evaluations of the same formulas (torch on the CPU) and against
+oracle/moe_oracle.py run in fp64 on the device's own logits.
+
+Bar: integer outputs bit-exact; floating point within rtol = atol = 1e-4 of the fp64 result (the
+absolute term times the tensor's rms where that exceeds 1) and 1e-5 norm-wise: two to three
+orders of magnitude inside the 1e-2 the benchmark definition allows the bf16 path (fp32 products
+summed in fp32 over at most a few thousand terms sit near 1e-6).
+"""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import moe_oracle as O
+
+pytestmark = pytest.mark.gpu
+RTOL = ATOL = 1e-4
+
+
+def _say(*a):
+    print(*a, flush=True)
+
+
+@pytest.fixture(scope="module")
+def P(pkg, lib):
+    assert torch.cuda.is_available(), "GPU tests need an MI355X"
+    return pkg
+
+
+def _close(name, got, ref, rtol=RTOL, atol=ATOL):
+    got, ref = got.double().cpu(), ref.double().cpu()
+    d = (got - ref).abs()
+    # element-wise with the absolute term scaled by the tensor's rms where that exceeds 1 (sums with
+    # cancellation carry the rounding of their large terms), and norm-wise at 1e-5
+    scale = max(1.0, ref.pow(2).mean().sqrt().item()) if d.numel() else 1.0
+    bad = (d > atol * scale + rtol * ref.abs()).double().mean().item() if d.numel() else 0.0
+    rel = (d.norm() / ref.norm().clamp_min(1e-30)).item()
+    _say(f"  {name}: max abs {d.max().item() if d.numel() else 0:.3e}  rel_fro {rel:.3e}  outside {bad:.2e}")
+    assert bad == 0.0 and rel <= 1e-5, name
+
+
+def _offsets(counts):
+    offs = np.zeros(len(counts) + 1, dtype=np.int32)
+    offs[1:] = np.cumsum(counts)
+    return offs
+
+
+@pytest.mark.parametrize("counts,N,K", [
+    ([64, 64, 64, 64], 64, 64),            # whole tiles
+    ([1, 0, 130, 63, 0, 65], 72, 40),      # ragged rows, empty experts, N and K off the tile sizes
+    ([0, 0, 5], 4, 4),                     # the smallest widths
+    ([300, 7, 0, 513, 64, 1, 0, 200], 516, 260),
+    ([0, 0, 0], 64, 64),                   # no rows at all
+])
+def test_f32_gemm_rows_and_wgrad(P, counts, N, K):
+    _say("f32 gemm", counts, N, K)
+    ops = P.ops
+    E, R = len(counts), int(sum(counts))
+    offs = _offsets(counts)
+    g = torch.Generator().manual_seed(R + N + K)
+    a = torch.randn(R, K, generator=g)
+    b_t = torch.randn(E, N, K, generator=g)      # used as a @ b[e].T
+    b_n = torch.randn(E, K, N, generator=g)      # used as a @ b[e]
+    c0 = torch.randn(R, N, generator=g)
+    offs_d = torch.from_numpy(offs).cuda()
+    ref_t = torch.zeros(R, N, dtype=torch.float64)
+    ref_n = torch.zeros(R, N, dtype=torch.float64)
+    for e in range(E):
+        s, t = int(offs[e]), int(offs[e + 1])
+        ref_t[s:t] = a[s:t].double() @ b_t[e].double().t()
+        ref_n[s:t] = a[s:t].double() @ b_n[e].double()
+    got_t = ops.f32_gemm_rows(a.cuda(), b_t.cuda(), offs_d, True)
+    got_n = ops.f32_gemm_rows(a.cuda(), b_n.cuda(), offs_d, False)
+    _close("a @ b^T", got_t, ref_t)
+    _close("a @ b", got_n, ref_n)
+    acc = c0.cuda().clone()
+    ops.f32_gemm_rows(a.cuda(), b_n.cuda(), offs_d, False, out=acc)
+    _close("c += a @ b", acc, c0.double() + ref_n)
+    # weight gradients: dw[e] = a[rows]^T @ c0[rows]; exact zeros for experts without rows
+    ref_w = torch.zeros(E, K, N, dtype=torch.float64)
+    for e in range(E):
+        s, t = int(offs[e]), int(offs[e + 1])
+        ref_w[e] = a[s:t].double().t() @ c0[s:t].double()
+    got_w = ops.f32_gemm_wgrad(a.cuda(), c0.cuda(), offs_d, E)
+    _close("dw", got_w, ref_w)
+    for e in range(E):
+        if counts[e] == 0:
+            assert got_w[e].abs().max().item() == 0.0
+    prev = torch.randn(E, K, N, generator=g)
+    acc_w = prev.cuda().clone()
+    ops.f32_gemm_wgrad(a.cuda(), c0.cuda(), offs_d, E, out=acc_w)
+    _close("dw accumulated", acc_w, prev.double() + ref_w)
+    for e in range(E):
+        if counts[e] == 0:
+            assert torch.equal(acc_w[e].cpu(), prev[e])
+
+
+@pytest.mark.parametrize("T,H,E,k", [(300, 64, 8, 2), (1000, 132, 64, 8), (5, 4, 3, 1), (64, 2048, 16, 4)])
+def test_f32_row_movers(P, T, H, E, k):
+    _say("f32 movers", T, H, E, k)
+    ops = P.ops
+    g = torch.Generator().manual_seed(T + H + E + k)
+    x = torch.randn(T, H, generator=g)
+    logits = torch.randn(T, E, generator=g)
+    ids, gates = ops.router_topk(logits.cuda(), k)
+    counts, offs, pos_to_row, row_to_pos = ops.histogram_scan(ids, E)
+    p2r, r2p = pos_to_row.cpu().long(), row_to_pos.cpu().long()
+    R = T * k
+    xp = ops.f32_gather_rows(x.cuda(), pos_to_row, k)
+    assert torch.equal(xp.cpu(), x[p2r // k])                       # a pure copy: bit-exact
+    y = torch.randn(R, H, generator=g)
+    out = ops.f32_combine_fwd(y.cuda(), gates, row_to_pos, T, k)
+    gc = gates.cpu().double()
+    ref_out = (y.double()[r2p] * gc.unsqueeze(-1)).view(T, k, H).sum(1)
+    _close("combine fwd", out, ref_out, rtol=1e-5, atol=1e-5)
+    dy = torch.randn(T, H, generator=g)
+    dyp, dgates = ops.f32_combine_bwd(dy.cuda(), y.cuda(), gates, pos_to_row, k)
+    _close("dyp", dyp, dy.double()[p2r // k] * gc[p2r].unsqueeze(-1), rtol=1e-6, atol=1e-6)
+    ref_dg = torch.zeros(R, dtype=torch.float64)
+    ref_dg[p2r] = (dy.double()[p2r // k] * y.double()).sum(-1)
+    _close("dgates", dgates, ref_dg, rtol=1e-5, atol=1e-4)
+    dyp2, none = ops.f32_combine_bwd(dy.cuda(), None, gates, pos_to_row, k)
+    assert none is None and torch.equal(dyp2, dyp)
+    dxp = torch.randn(R, H, generator=g)
+    dx = ops.f32_permute_bwd(dxp.cuda(), row_to_pos, T, k)
+    _close("permute bwd", dx, dxp.double()[r2p].view(T, k, H).sum(1), rtol=1e-5, atol=1e-5)
+
+
+def test_f32_swiglu_matches_autograd(P):
+    ops = P.ops
+    g_ = torch.Generator().manual_seed(5)
+    g = (torch.randn(333, 68, generator=g_) * 3).double().requires_grad_(True)
+    u = torch.randn(333, 68, generator=g_).double().requires_grad_(True)
+    dact = torch.randn(333, 68, generator=g_).double()
+    act = F.silu(g) * u
+    act.backward(dact)
+    got = ops.f32_swiglu(g.detach().float().cuda(), u.detach().float().cuda())
+    _close("act", got, act.detach(), rtol=1e-5, atol=1e-6)
+    dg, du = ops.f32_swiglu_bwd(dact.float().cuda(), g.detach().float().cuda(), u.detach().float().cuda())
+    _close("dg", dg, g.grad, rtol=1e-5, atol=1e-5)
+    _close("du", du, u.grad, rtol=1e-5, atol=1e-5)
+
+
+def _layer_case(P, T, H, I, E, k, seed, bias=False):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(T, H, generator=g)
+    wr = torch.randn(E, H, generator=g) * 0.3
+    w1 = torch.randn(E, I, H, generator=g) * 0.1
+    w3 = torch.randn(E, I, H, generator=g) * 0.1
+    w2 = torch.randn(E, H, I, generator=g) * 0.1
+    dy = torch.randn(T, H, generator=g)
+    b = (torch.randn(E, generator=g) if bias else None)
+    return x, wr, w1, w3, w2, dy, b
+
+
+@pytest.mark.parametrize("T,H,I,E,k,bias", [
+    (2048, 1024, 512, 8, 2, False),     # benchmark config 1's shape
+    (700, 132, 68, 16, 4, True),        # nothing a multiple of a tile, a router bias
+    (64, 64, 64, 64, 8, False),         # most experts empty or nearly so
+])
+def test_f32_layer_matches_the_oracle_in_fp64(P, T, H, I, E, k, bias):
+    """moe_ffn_f32 on fp32 tensors against the oracle evaluated in fp64 on the same fp32 values
+    and the device's own fp32 logits: integer routing outputs bit-exact, every floating point
+    result (out, dx, dlogits, the three weight gradients, the bias gradient) within 1e-4."""
+    _say("f32 layer", T, H, I, E, k, bias)
+    x, wr, w1, w3, w2, dy, b = _layer_case(P, T, H, I, E, k, seed=T + H + E, bias=bias)
+    dev = "cuda"
+    xd = x.to(dev).requires_grad_(True)
+    ws = [w.to(dev).requires_grad_(True) for w in (w1, w3, w2)]
+    logits = F.linear(x.to(dev), wr.to(dev)).requires_grad_(True)
+    bd = b.to(dev).requires_grad_(True) if bias else None
+    out, routing = P.moe_ffn_f32(xd, logits, *ws, k, bias=bd, return_routing=True)
+    assert out.dtype == torch.float32
+    out.backward(dy.to(dev))
+    lg = logits.detach().cpu()
+    f = O.moe_forward(x, wr, w1, w3, w2, k, logits=((lg + b).double() if bias else lg.double()),
+                      compute_dtype=torch.float64)
+    assert np.array_equal(routing["ids"].cpu().numpy().reshape(T, k), f["ids"].astype(np.int32))
+    assert np.array_equal(routing["counts"].cpu().numpy(), f["counts"].astype(np.int32))
+    assert np.array_equal(routing["offs"].cpu().numpy(), f["starts"].astype(np.int32))
+    assert np.array_equal(routing["pos_to_row"].cpu().numpy(), f["pos_to_row"].astype(np.int32))
+    assert np.array_equal(routing["row_to_pos"].cpu().numpy(), f["row_to_pos"].astype(np.int32))
+    bk = O.moe_backward(f, dy, wr, w1, w3, w2)
+    _close("out", out, f["out"])
+    _close("dx (expert path)", xd.grad, bk["dx_expert"])
+    _close("dlogits", logits.grad, bk["dlogits"])
+    for name, w in zip(("dw1", "dw3", "dw2"), ws):
+        _close(name, w.grad, bk[name])
+    if bias:
+        _close("dbias", bd.grad, bk["dlogits"].sum(0))
+    # the same call on the bf16 matrix cores is two orders of magnitude further away
+    out_bf, _ = P.routed_moe(x.to(dev), wr.to(dev), w1.to(dev), w3.to(dev), w2.to(dev), k) if not bias else (None, None)
+    if out_bf is not None:
+        e32 = (out.double().cpu() - f["out"]).norm() / f["out"].norm()
+        e16 = (out_bf.double().cpu() - f["out"]).norm() / f["out"].norm()
+        _say(f"  rel error of out: fp32 path {e32:.2e}, bf16 path {e16:.2e}")
+        assert e32 * 20 < e16
+
+
+def test_module_runs_in_fp32_when_the_reference_would(P):
+    """fp32 parameters, fp32 input, no autocast: fp32 from end to end (fp32 logits from the
+    module's own nn.Linear, fp32 experts), checked against the differentiable restatement of mlp.py:100-167
+    in fp64 (and the forward against the literal padded-bmm one).  Under bf16 autocast, with bf16 input, or with
+    `bf16_compute_for_fp32_calls` the same module takes the bf16 path."""
+    cfg = P.ModelConfig(hidden_size=128, num_experts=8, num_experts_per_tok=2, moe_intermediate_size=64,
+                        init_std=0.05)
+    m = P.MoE(cfg, 2)
+    B, T, H = 2, 100, 128
+    g = torch.Generator().manual_seed(12)
+    x = torch.randn(B, T, H, generator=g).cuda().requires_grad_(True)
+    dy = torch.randn(B, T, H, generator=g).cuda()
+    assert m._runs_in_fp32(x)
+    out, gate_logits = m(x)
+    assert out.dtype == torch.float32 and gate_logits.dtype == torch.float32
+    out.backward(dy)
+    params = dict(wr=m.router.weight, w1=m.experts_gate_weights, w3=m.experts_up_weights,
+                  w2=m.experts_down_weights)
+    c = {n: p.detach().cpu().double().requires_grad_(True) for n, p in params.items()}
+    xr = x.detach().cpu().double().requires_grad_(True)
+    # (the selection is taken from the device's fp32 logits: a near-tie could fall the other way
+    # in fp64, and that the device selects by the canonical rule is tested on its own)
+    ids, _ = O.topk_select(gate_logits.detach().cpu().reshape(-1, 8), 2)
+    ref_out = O.moe_forward_autograd(xr.reshape(-1, H), c["wr"], c["w1"], c["w3"], c["w2"], 2, ids=ids)
+    ref_out.backward(dy.cpu().double().reshape(-1, H))
+    _close("out", out.reshape(-1, H), ref_out.detach())
+    _close("gate_logits", gate_logits.reshape(-1, 8), F.linear(xr.detach().reshape(-1, H), c["wr"].detach()),
+           rtol=1e-5, atol=1e-5)
+    lit = O.moe_forward_padded_bmm(xr.detach().reshape(-1, H), c["wr"].detach(), c["w1"].detach(),
+                                   c["w3"].detach(), c["w2"].detach(), 2,
+                                   logits=gate_logits.detach().cpu().double().reshape(-1, 8))
+    _close("out vs the padded-bmm restatement", out.reshape(-1, H), lit, rtol=1e-4, atol=1e-4)
+    _close("dx", x.grad.reshape(-1, H), xr.grad.reshape(-1, H))
+    for n, p in params.items():
+        assert p.grad.dtype == torch.float32
+        _close("d" + n, p.grad, c[n].grad)
+    # the other calling conventions keep the bf16 path
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        assert not m._runs_in_fp32(x)
+    assert not m._runs_in_fp32(x.detach().to(torch.bfloat16))
+    m.bf16_compute_for_fp32_calls = True
+    assert not m._runs_in_fp32(x)
+    out_bf, _ = m(x.detach())
+    assert out_bf.dtype == torch.float32
+    rel = ((out_bf - out.detach()).norm() / out.detach().norm()).item()
+    _say(f"  bf16 compute on the same fp32 call: rel diff {rel:.2e}")
+    assert 1e-4 < rel < 2e-2
+    # forward_prenorm falls back to the separate calls for an fp32 call
+    m.bf16_compute_for_fp32_calls = False
+    norm = torch.nn.Module()
+    norm.weight = torch.nn.Parameter(torch.ones(H, device="cuda"))
+    norm.variance_epsilon = 1e-6
+    norm.forward = lambda t: t * torch.rsqrt(t.pow(2).mean(-1, keepdim=True) + 1e-6) * norm.weight
+    y2, lg2 = m.forward_prenorm(x.detach(), norm)
+    y1, lg1 = m(norm(x.detach()))
+    assert torch.equal(y2, x.detach() + y1) and torch.equal(lg2, lg1)

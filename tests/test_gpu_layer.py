@@ -833,13 +833,15 @@ def test_backward_twice_through_a_retained_graph(P, entry):
         assert torch.equal(t.grad, o * 2)
 
 
-def test_module_called_in_fp32_without_autocast(P):
-    """fp32 parameters, fp32 input, no autocast: the router product is the fp32 `nn.Linear`
-    product (fp32 logits, so the selection follows fp32 values), the experts still compute in
-    bf16 on the matrix cores; outputs and every gradient are fp32."""
+def test_module_called_in_fp32_without_autocast_on_the_bf16_cores(P):
+    """fp32 parameters, fp32 input, no autocast, `bf16_compute_for_fp32_calls` set: the router
+    product is the fp32 `nn.Linear` product (fp32 logits, so the selection follows fp32 values),
+    the experts compute in bf16 on the matrix cores; outputs and every gradient are fp32.
+    (Without the switch such a call runs in fp32 from end to end: tests/test_gpu_f32.py.)"""
     cfg = P.ModelConfig(hidden_size=128, num_experts=8, num_experts_per_tok=2, moe_intermediate_size=64,
                         init_std=0.05)
     m = P.MoE(cfg, 2)
+    m.bf16_compute_for_fp32_calls = True
     B, T, H = 2, 100, 128
     g = torch.Generator().manual_seed(12)
     x = torch.randn(B, T, H, generator=g).cuda().requires_grad_(True)

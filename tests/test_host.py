@@ -34,7 +34,7 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(cdll, n), n
     assert sorted(names) == sorted(pkg.lib.SIGNATURES)
     L = pkg.lib.load()
-    assert L.abi_version == 100
+    assert L.abi_version == 101
     assert L.cdll.moe_dispatch_workspace_bytes(1000, 8) == 4 * (8 + 1) * 4
 
 
@@ -167,6 +167,7 @@ _OPTIONAL_POINTERS = {
     "moe_combine_fwd": {"gates"}, "moe_combine_fwd_residual": {"gates"},
     "moe_combine_bwd": {"gates"}, "moe_combine_bwd_by_token": {"gates"},
     "moe_rmsnorm_bwd": {"d2", "dres"},
+    "moe_f32_combine_bwd": {"y", "dgates"},
 }
 
 

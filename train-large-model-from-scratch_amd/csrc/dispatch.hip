@@ -547,7 +547,7 @@ inline unsigned mover_grid(int64_t rows, int per_block) {
 
 }  // namespace
 
-extern "C" int moe_abi_version(void) { return 100; }
+extern "C" int moe_abi_version(void) { return 101; }
 
 extern "C" int64_t moe_dispatch_workspace_bytes(int64_t R, int64_t E) {
   if (R < 0 || E <= 0) return 0;

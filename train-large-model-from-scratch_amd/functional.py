@@ -17,10 +17,11 @@
                gradient streams into x (expert path, router path, residual) meet inside the
                normalisation's backward kernel instead of in separate additions.
 
-`moe_ffn` and `experts_rows` always compute in bf16 on the matrix cores with fp32
-accumulation, whatever the input dtype; outputs and input gradients take the dtype of `x`,
-weight gradients the dtype of the weights.  There is no host synchronisation anywhere in
-either direction.
+`moe_ffn` and `experts_rows` compute in bf16 on the matrix cores with fp32 accumulation,
+whatever the input dtype; outputs and input gradients take the dtype of `x`, weight gradients
+the dtype of the weights.  `moe_ffn_f32` is the same function with every step in fp32 (fp32
+matrix instructions, fp32 rows): what the reference computes when it is called without autocast
+on fp32 tensors.  There is no host synchronisation anywhere in either direction.
 
 Weight gradients into `.grad` (`accumulate_into_grad=True`): the reference's trainer sums
 the gradients of several micro-steps in the parameters' `.grad` (training/trainer.py:241-248),
@@ -308,6 +309,75 @@ def moe_ffn(x: torch.Tensor, logits: torch.Tensor, w1: torch.Tensor, w3: torch.T
         grad_params = tuple(w if (w.requires_grad and w.is_leaf) else None for w in (w1, w3, w2))
     out, ids, gates, counts, offs, pos_to_row, row_to_pos = _MoEFFN.apply(
         x, logits, w1, w3, w2, k, bias, bf16_weights, grad_params)
+    if return_routing:
+        return out, {"ids": ids, "gates": gates, "counts": counts, "offs": offs,
+                     "pos_to_row": pos_to_row, "row_to_pos": row_to_pos}
+    return out
+
+
+class _MoEFFNf32(torch.autograd.Function):
+    """The fp32 path: model/modules/mlp.py:101-167 with fp32 operands and no autocast."""
+
+    @staticmethod
+    def forward(ctx, x, logits, w1, w3, w2, k, bias):
+        T, H = x.shape
+        E = logits.shape[1]
+        x, logits = _dense(x), _dense(logits)
+        w1, w3, w2 = _dense(w1), _dense(w3), _dense(w2)
+        ids, gates = ops.router_topk(logits, k, bias)
+        counts, offs, pos_to_row, row_to_pos = ops.histogram_scan(ids, E)
+        xp = ops.f32_gather_rows(x, pos_to_row, k)
+        g = ops.f32_gemm_rows(xp, w1, offs, True)
+        u = ops.f32_gemm_rows(xp, w3, offs, True)
+        act = ops.f32_swiglu(g, u)
+        y = ops.f32_gemm_rows(act, w2, offs, True)
+        out = ops.f32_combine_fwd(y, gates, row_to_pos, T, k)
+        if any(ctx.needs_input_grad):
+            ctx.save_for_backward(xp, g, u, act, y, gates, ids, offs, pos_to_row, row_to_pos, w1, w3, w2)
+        ctx.k, ctx.E = k, E
+        ctx.mark_non_differentiable(ids, gates, counts, offs, pos_to_row, row_to_pos)
+        ctx.set_materialize_grads(False)
+        ctx.out_shape = out.shape
+        return out, ids, gates, counts, offs, pos_to_row, row_to_pos
+
+    @staticmethod
+    def backward(ctx, dout, *unused):
+        xp, g, u, act, y, gates, ids, offs, pos_to_row, row_to_pos, w1, w3, w2 = ctx.saved_tensors
+        k, E = ctx.k, ctx.E
+        if dout is None:
+            dout = torch.zeros(ctx.out_shape, dtype=torch.float32, device=xp.device)
+        T = dout.shape[0]
+        need = ctx.needs_input_grad
+        dyp, dgates = ops.f32_combine_bwd(_dense(dout.float()), y if (need[1] or need[6]) else None, gates,
+                                          pos_to_row, k)
+        dact = ops.f32_gemm_rows(dyp, w2, offs, False)
+        dg, du = ops.f32_swiglu_bwd(dact, g, u)
+        dx = None
+        if need[0]:
+            dxp = ops.f32_gemm_rows(dg, w1, offs, False)
+            ops.f32_gemm_rows(du, w3, offs, False, out=dxp)
+            dx = ops.f32_permute_bwd(dxp, row_to_pos, T, k)
+        dw1 = ops.f32_gemm_wgrad(dg, xp, offs, E) if need[2] else None
+        dw3 = ops.f32_gemm_wgrad(du, xp, offs, E) if need[3] else None
+        dw2 = ops.f32_gemm_wgrad(dyp, act, offs, E) if need[4] else None
+        dlogits = dbias = None
+        if need[1] or need[6]:
+            dlogits = ops.router_topk_bwd(gates, dgates, ids, T, E, k, torch.float32)
+            dbias = dlogits.sum(0) if need[6] else None
+            if not need[1]:
+                dlogits = None
+        return dx, dlogits, dw1, dw3, dw2, None, dbias
+
+
+def moe_ffn_f32(x: torch.Tensor, logits: torch.Tensor, w1: torch.Tensor, w3: torch.Tensor,
+                w2: torch.Tensor, k: int, bias: torch.Tensor | None = None, return_routing: bool = False):
+    """`moe_ffn` with every tensor and every product in fp32 (all arguments fp32; H and the FFN
+    width multiples of 4).  Routing, counts and the permutation are the same kernels and the same
+    bits as in `moe_ffn` given the same logits."""
+    for name, t in (("x", x), ("logits", logits), ("w1", w1), ("w3", w3), ("w2", w2)):
+        if t.dtype != torch.float32:
+            raise TypeError(f"moe_ffn_f32: {name} must be fp32, got {t.dtype}")
+    out, ids, gates, counts, offs, pos_to_row, row_to_pos = _MoEFFNf32.apply(x, logits, w1, w3, w2, k, bias)
     if return_routing:
         return out, {"ids": ids, "gates": gates, "counts": counts, "offs": offs,
                      "pos_to_row": pos_to_row, "row_to_pos": row_to_pos}

@@ -58,6 +58,14 @@ SIGNATURES = {
                                _i64, _vp]),
     "moe_combine_bwd_by_token": (_int, [_vp, _int, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _vp]),
     "moe_cast_f32_bf16": (_int, [_vp, _vp, _i64, _vp]),
+    "moe_f32_gather_rows": (_int, [_vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp]),
+    "moe_f32_combine_fwd": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp]),
+    "moe_f32_combine_bwd": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _vp]),
+    "moe_f32_permute_bwd": (_int, [_vp, _vp, _i64, _i64, _i64, _vp, _vp]),
+    "moe_f32_swiglu_fwd": (_int, [_vp, _vp, _i64, _vp, _vp]),
+    "moe_f32_swiglu_bwd": (_int, [_vp, _vp, _vp, _i64, _vp, _vp, _vp]),
+    "moe_f32_gemm_rows": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp, _int, _vp]),
+    "moe_f32_gemm_wgrad": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _int, _vp]),
 }
 
 ERRORS = {-1: "MOE_ERR_NULL", -2: "MOE_ERR_SHAPE", -3: "MOE_ERR_LIMIT", -4: "MOE_ERR_DTYPE",

@@ -12,7 +12,7 @@ import torch.nn as nn
 from torch.optim.optimizer import register_optimizer_step_post_hook
 
 from . import ops, parallel_state, traced
-from .functional import moe_ffn, prenorm_moe, routed_moe, router_linear
+from .functional import moe_ffn, moe_ffn_f32, prenorm_moe, routed_moe, router_linear
 
 
 # Number of optimizer steps taken in this process, counted by a global post-step hook of
@@ -76,6 +76,11 @@ class MoE(nn.Module):
         # `forward` uses) instead of the fused norm+router kernel, whose summation order can move
         # a bf16 logit by one unit in the last place and with it the routing of a near-tie.
         self.fused_router = True
+        # False (the reference's rule): a call without autocast on fp32 input and fp32 parameters
+        # computes in fp32 from end to end, as the reference's bmm's then do (mlp.py:154-157).
+        # True: such a call runs on the bf16 matrix cores like every other one (fp32 in and out,
+        # bf16 operands, fp32 accumulation): about 20 times the throughput at bf16 precision.
+        self.bf16_compute_for_fp32_calls = False
         self._init_expert_weights(config.seed)
 
     def _init_expert_weights(self, base_seed: int):
@@ -166,8 +171,27 @@ class MoE(nn.Module):
         return (x.is_cuda and torch.is_autocast_enabled("cuda")
                 and torch.get_autocast_dtype("cuda") == torch.bfloat16)
 
+    def _runs_in_fp32(self, x: torch.Tensor) -> bool:
+        """Whether the reference would run this call in fp32: fp32 input, fp32 parameters, no
+        autocast."""
+        if self.bf16_compute_for_fp32_calls or x.dtype != torch.float32:
+            return False
+        if x.is_cuda and torch.is_autocast_enabled("cuda"):
+            return False
+        return all(w.dtype == torch.float32 for w in (self.router.weight, self.experts_gate_weights,
+                                                      self.experts_up_weights, self.experts_down_weights))
+
+    @torch._dynamo.disable
+    def _experts_f32(self, x2d: torch.Tensor, logits2d: torch.Tensor) -> torch.Tensor:
+        return moe_ffn_f32(x2d, logits2d, self.experts_gate_weights, self.experts_up_weights,
+                           self.experts_down_weights, self.top_k)
+
     def forward(self, x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
         B, T, D = x.size()
+        if not torch.compiler.is_compiling() and self._runs_in_fp32(x):
+            gate_logits = self.router(x)  # fp32 product and fp32 gradients, as nn.Linear gives them
+            out = self._experts_f32(x.reshape(B * T, D), gate_logits.reshape(B * T, self.num_experts))
+            return out.reshape(B, T, D), gate_logits
         if torch.compiler.is_compiling():
             # under torch.compile (trainer.py:130-131): the same kernels as registered
             # operators the tracer can keep in the graph (traced.py); no cached weight copies
@@ -199,9 +223,10 @@ class MoE(nn.Module):
         calling the three pieces separately under bf16 autocast; the residual stream is read
         once on the way in and written once on the way out."""
         B, T, D = x.size()
-        if D > 8192 or self._router_has_hooks():
-            # wider than the fused norm kernels hold in registers, or hooks on the router that only
-            # a call of the nn.Linear runs: the separate calls
+        if D > 8192 or self._router_has_hooks() or self._runs_in_fp32(x):
+            # wider than the fused norm kernels hold in registers, hooks on the router that only a
+            # call of the nn.Linear runs, or an fp32 call (the norm then is the caller's fp32
+            # module): the separate calls
             out, logits = self(norm(x))
             return (x + out if add_residual else out), logits
         out, logits = prenorm_moe(x.reshape(B * T, D), norm.weight, self.router.weight,

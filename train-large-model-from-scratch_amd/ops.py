@@ -376,3 +376,91 @@ def cast_bf16(w: torch.Tensor) -> torch.Tensor:
     out = torch.empty(w.shape, dtype=torch.bfloat16, device=w.device)
     _lib.load().call("moe_cast_f32_bf16", _p(w), _p(out), w.numel(), _stream())
     return out
+
+
+# ---- the path in fp32 (layer called without autocast on fp32 tensors) ---------------------------
+
+def _f32(*ts):
+    for t in ts:
+        if t is not None and t.dtype != torch.float32:
+            raise TypeError(f"the fp32 entry points take fp32 tensors, got {t.dtype}")
+
+
+def f32_gather_rows(x: torch.Tensor, pos_to_row: torch.Tensor, k: int) -> torch.Tensor:
+    """xp[pos] = x[pos_to_row[pos] // k], fp32 [R,H]."""
+    _f32(x)
+    T, H = x.shape
+    R = pos_to_row.numel()
+    xp = torch.empty(R, H, dtype=torch.float32, device=x.device)
+    _lib.load().call("moe_f32_gather_rows", _p(x), _p(pos_to_row), T, R, H, k, _p(xp), _stream())
+    return xp
+
+
+def f32_combine_fwd(y: torch.Tensor, gates: torch.Tensor, row_to_pos: torch.Tensor, T: int, k: int):
+    _f32(y, gates)
+    H = y.shape[-1]
+    out = torch.empty(T, H, dtype=torch.float32, device=y.device)
+    _lib.load().call("moe_f32_combine_fwd", _p(y), _p(gates), _p(row_to_pos), T, H, k, _p(out), _stream())
+    return out
+
+
+def f32_combine_bwd(dy, y, gates, pos_to_row, k: int):
+    """-> dyp fp32 [R,H], dgates fp32 [R] (None when y is None)."""
+    _f32(dy, y, gates)
+    T, H = dy.shape
+    R = pos_to_row.numel()
+    dyp = torch.empty(R, H, dtype=torch.float32, device=dy.device)
+    dgates = torch.empty(R, dtype=torch.float32, device=dy.device) if y is not None else None
+    _lib.load().call("moe_f32_combine_bwd", _p(dy), _p(y), _p(gates), _p(pos_to_row), T, R, H, k, _p(dyp),
+                     _p(dgates), _stream())
+    return dyp, dgates
+
+
+def f32_permute_bwd(dxp: torch.Tensor, row_to_pos: torch.Tensor, T: int, k: int) -> torch.Tensor:
+    _f32(dxp)
+    H = dxp.shape[-1]
+    dx = torch.empty(T, H, dtype=torch.float32, device=dxp.device)
+    _lib.load().call("moe_f32_permute_bwd", _p(dxp), _p(row_to_pos), T, H, k, _p(dx), _stream())
+    return dx
+
+
+def f32_swiglu(g: torch.Tensor, u: torch.Tensor) -> torch.Tensor:
+    _f32(g, u)
+    act = torch.empty_like(g)
+    _lib.load().call("moe_f32_swiglu_fwd", _p(g), _p(u), g.numel(), _p(act), _stream())
+    return act
+
+
+def f32_swiglu_bwd(dact, g, u):
+    _f32(dact, g, u)
+    dg, du = torch.empty_like(g), torch.empty_like(g)
+    _lib.load().call("moe_f32_swiglu_bwd", _p(dact), _p(g), _p(u), g.numel(), _p(dg), _p(du), _stream())
+    return dg, du
+
+
+def f32_gemm_rows(a: torch.Tensor, b: torch.Tensor, offs: torch.Tensor, transpose_b: bool,
+                  out: torch.Tensor | None = None) -> torch.Tensor:
+    """Per expert e over its rows: a[rows] @ b[e].T (`transpose_b`, b [E,N,K]) or a[rows] @ b[e]
+    (b [E,K,N]).  With `out` the product is added into it."""
+    _f32(a, b, out)
+    R, K = a.shape
+    E = b.shape[0]
+    N = b.shape[1] if transpose_b else b.shape[2]
+    if (b.shape[2] if transpose_b else b.shape[1]) != K:
+        raise ValueError(f"depth mismatch: a {tuple(a.shape)}, b {tuple(b.shape)}, transpose_b={transpose_b}")
+    c = out if out is not None else torch.empty(R, N, dtype=torch.float32, device=a.device)
+    _lib.load().call("moe_f32_gemm_rows", _p(a), _p(b), _p(offs), E, R, N, K, int(transpose_b), _p(c),
+                     int(out is not None), _stream())
+    return c
+
+
+def f32_gemm_wgrad(a: torch.Tensor, b: torch.Tensor, offs: torch.Tensor, E: int,
+                   out: torch.Tensor | None = None) -> torch.Tensor:
+    """dw[e] = a[rows of e].T @ b[rows of e] -> fp32 [E,M,N]; with `out` added into it."""
+    _f32(a, b, out)
+    R, M = a.shape
+    N = b.shape[1]
+    dw = out if out is not None else torch.empty(E, M, N, dtype=torch.float32, device=a.device)
+    _lib.load().call("moe_f32_gemm_wgrad", _p(a), _p(b), _p(offs), E, R, M, N, _p(dw), int(out is not None),
+                     _stream())
+    return dw
