@@ -406,6 +406,59 @@ def module_config3(P, torch, dev, steps, warmup):
             "entry": "MoE.forward", **out}
 
 
+MFMA_F32_PEAK_TFLOPS = 157.3     # MI355X dense fp32 matrix
+
+
+def fp32_config3(P, torch, dev, steps=3, warmup=1):
+    """Configuration 3 in fp32 from end to end (`moe_ffn_f32`: what the reference computes when its
+    layer is called without autocast on fp32 tensors), priced against the fp32 matrix peak."""
+    s = P.configs.SHAPES[3]
+    inp = P.configs.make_inputs(3)
+    x = inp["x"].float().to(dev).requires_grad_(True)
+    wr = inp["wr"].float().to(dev)
+    ws = [inp[n].float().to(dev).requires_grad_(True) for n in ("w1", "w3", "w2")]
+    dy = inp["dy"].float().to(dev)
+    logits = torch.nn.functional.linear(x.detach(), wr).requires_grad_(True)
+    leaves = (x, logits, *ws)
+
+    def step():
+        for t in leaves:
+            t.grad = None
+        P.moe_ffn_f32(x, logits, *ws, s.k).backward(dy)
+
+    ms, ms_median, ms_min = _timed_steps(torch, step, steps, warmup)
+    flops = P.configs.gemm_flops(s)
+    watch = _LaunchEvents(torch)
+    P.lib.load().observer = watch
+    try:
+        step()
+        torch.cuda.synchronize()
+    finally:
+        P.lib.load().observer = None
+    per = {"moe_f32_gemm_rows": 2, "moe_f32_gemm_wgrad": 2}  # flops per launch in units of R*H*I
+    recs, g_ms = [], 0.0
+    for name, kms in watch.per_launch_ms(1):
+        rec = {"entry": name, "ms": round(kms, 4)}
+        if name in per and kms > 0:
+            tf = per[name] * s.R * s.H * s.I / kms / 1e9
+            rec.update(achieved=round(tf, 1), unit="TFLOP/s", frac=round(tf / MFMA_F32_PEAK_TFLOPS, 4))
+            g_ms += kms
+        recs.append(rec)
+    dom = max((r for r in recs if "frac" in r), key=lambda r: r["ms"])
+    roof = {"kernel": dom["entry"].replace("moe_", "", 1), "bound": "mfma", "achieved": dom["achieved"],
+            "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": dom["frac"], "traffic": None, "ms": dom["ms"],
+            "measured": "HIP events around this launch in one step that follows the timed ones",
+            "all_gemms_tflops": round(flops / g_ms / 1e9, 1),
+            "all_gemms_frac": round(flops / g_ms / 1e9 / MFMA_F32_PEAK_TFLOPS, 4)}
+    del x, ws, dy, logits, leaves
+    torch.cuda.empty_cache()
+    return {"config": 3, "workload": s.name + ", every tensor and every product in fp32 (no autocast)",
+            "entry": "moe_ffn_f32", "dtype": "f32", "ms_per_step": round(ms, 4),
+            "ms_per_step_median": round(ms_median, 4), "ms_per_step_min": round(ms_min, 4),
+            "tflops": round(flops / ms / 1e9, 1), "fp32_matrix_peak_frac": round(flops / ms / 1e9 / MFMA_F32_PEAK_TFLOPS, 4),
+            "tokens_per_s": round(s.T / (ms * 1e-3), 1), "steps": steps, "roofline": roof, "kernels_in_step": recs}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -651,6 +704,7 @@ def main():
                 rec["cpu_baseline"] = cpu_leg(P, torch, cid, fraction)
             others.append(rec)
         others.append(module_config3(P, torch, dev, max(args.steps // 2, 5), args.warmup))
+        others.append(fp32_config3(P, torch, dev))
         blk = bench_block(args, torch, P, dev, steps=max(args.steps // 2, 5), warmup=3, cpu=not args.no_cpu)
         others.append({"config": 5, "workload": blk["config"]["workload"], "entry": "Block.forward",
                        "ms_per_step": blk["ms_per_step"], "tokens_per_s": blk["value"],
