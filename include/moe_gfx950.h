@@ -328,7 +328,8 @@ int moe_cast_f32_bf16(const float* src, uint16_t* dst, int64_t n, void* stream);
 /* mlp.py:104-131 (repeat_interleave + both sorts): xp[pos,:] = x[pos_to_row[pos] / k, :]. */
 int moe_f32_gather_rows(const float* x, const int32_t* pos_to_row, int64_t T, int64_t R, int64_t H,
                         int64_t k, float* xp, void* stream);
-/* mlp.py:160-169: out[t,:] = sum_j gates[t*k+j] * y[row_to_pos[t*k+j],:], j ascending. */
+/* mlp.py:160-169: out[t,:] = sum_j gates[t*k+j] * y[row_to_pos[t*k+j],:], j ascending.
+ * gates may be NULL (all ones; with k = 1 a pure un-permute), here and in the backward. */
 int moe_f32_combine_fwd(const float* y, const float* gates, const int32_t* row_to_pos, int64_t T,
                         int64_t H, int64_t k, float* out, void* stream);
 /* Its backward: dyp[pos,:] = gates[row] * dy[row / k,:] and, unless dgates is NULL,

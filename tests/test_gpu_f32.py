@@ -255,3 +255,36 @@ def test_module_runs_in_fp32_when_the_reference_would(P):
     y2, lg2 = m.forward_prenorm(x.detach(), norm)
     y1, lg1 = m(norm(x.detach()))
     assert torch.equal(y2, x.detach() + y1) and torch.equal(lg2, lg1)
+
+
+def test_f32_rows_entry_matches_the_oracle_in_fp64(P):
+    """The post-dispatch entry in fp32 (`experts_rows_f32`: rows already on their rank + local
+    expert ids, a skewed load with two empty experts) against the oracle in fp64."""
+    R, H, I, E = 1500, 132, 68, 8
+    g = torch.Generator().manual_seed(21)
+    rows = torch.randn(R, H, generator=g)
+    w1 = torch.randn(E, I, H, generator=g) * 0.1
+    w3 = torch.randn(E, I, H, generator=g) * 0.1
+    w2 = torch.randn(E, H, I, generator=g) * 0.1
+    dout = torch.randn(R, H, generator=g)
+    p = torch.tensor([0.4, 0.0, 0.3, 0.05, 0.0, 0.15, 0.05, 0.05])
+    ids = torch.multinomial(p, R, replacement=True, generator=g)
+    rd = rows.cuda().requires_grad_(True)
+    ws = [w.cuda().requires_grad_(True) for w in (w1, w3, w2)]
+    out, routing = P.experts_rows_f32(rd, ids.cuda(), *ws, return_routing=True, check_ids=True)
+    out.backward(dout.cuda())
+    f = O.experts_rows_forward(rows, ids.numpy(), w1, w3, w2, compute_dtype=torch.float64)
+    b = O.experts_rows_backward(f, dout, w1, w3, w2)
+    assert np.array_equal(routing["counts"].cpu().numpy(), f["counts"].astype(np.int32))
+    assert np.array_equal(routing["pos_to_row"].cpu().numpy(), f["pos_to_row"].astype(np.int32))
+    _close("out", out, f["out"])
+    _close("drows", rd.grad, b["drows"])
+    for name, w in zip(("dw1", "dw3", "dw2"), ws):
+        _close(name, w.grad, b[name])
+        assert w.grad[1].abs().max().item() == 0.0 and w.grad[4].abs().max().item() == 0.0
+    with pytest.raises(ValueError):
+        bad = ids.clone()
+        bad[7] = E
+        P.experts_rows_f32(rows.cuda(), bad.cuda(), w1.cuda(), w3.cuda(), w2.cuda(), check_ids=True)
+    with pytest.raises(TypeError):
+        P.experts_rows_f32(rows.cuda().bfloat16(), ids.cuda(), w1.cuda(), w3.cuda(), w2.cuda())

@@ -177,7 +177,8 @@ __global__ __launch_bounds__(256) void f32_gather_rows_kernel(const float* __res
   }
 }
 
-// out[t, :] = sum_j gates[t*k+j] * y[row_to_pos[t*k+j], :], j ascending  (mlp.py:160-169)
+// out[t, :] = sum_j gates[t*k+j] * y[row_to_pos[t*k+j], :], j ascending  (mlp.py:160-169);
+// gates == nullptr: all ones (with k = 1 a pure un-permute)
 __global__ __launch_bounds__(256) void f32_combine_fwd_kernel(const float* __restrict__ y,
                                                               const float* __restrict__ gates,
                                                               const int32_t* __restrict__ row_to_pos, int R,
@@ -188,7 +189,7 @@ __global__ __launch_bounds__(256) void f32_combine_fwd_kernel(const float* __res
     for (int j = 0; j < k; ++j) {
       const int pos = row_to_pos[t * k + j];
       if (pos < 0 || pos >= R) continue;
-      const float g = gates[t * k + j];
+      const float g = gates ? gates[t * k + j] : 1.f;
       const f32x4 v = *reinterpret_cast<const f32x4*>(y + (long long)pos * H + h);
       acc += g * v;
     }
@@ -209,7 +210,7 @@ __global__ __launch_bounds__(256) void f32_combine_bwd_kernel(const float* __res
   const int row = pos_to_row[pos];
   const int t = row / k;
   const bool ok = row >= 0 && t < T;
-  const float g = ok ? gates[row] : 0.f;
+  const float g = ok ? (gates ? gates[row] : 1.f) : 0.f;
   float dot = 0.f;
   for (int h = threadIdx.x * 4; h < H; h += 256 * 4) {
     f32x4 d = {0.f, 0.f, 0.f, 0.f};
@@ -309,7 +310,7 @@ extern "C" int moe_f32_combine_fwd(const float* y, const float* gates, const int
   if (T == 0) return 0;
   MOE_CHECK_PTR(y);
   MOE_CHECK_PTR(out);
-  if (!gates || !row_to_pos) return MOE_ERR_NULL;
+  if (!row_to_pos) return MOE_ERR_NULL;
   hipLaunchKernelGGL(f32_combine_fwd_kernel, dim3((unsigned)T), dim3(256), 0, (hipStream_t)stream, y, gates,
                      row_to_pos, (int)(T * k), (int)H, (int)k, out);
   return moe_launch_status();
@@ -324,7 +325,7 @@ extern "C" int moe_f32_combine_bwd(const float* dy, const float* y, const float*
   if (R == 0) return 0;
   MOE_CHECK_PTR(dy);
   MOE_CHECK_PTR(dyp);
-  if (!gates || !pos_to_row) return MOE_ERR_NULL;
+  if (!pos_to_row) return MOE_ERR_NULL;
   if (dgates) MOE_CHECK_PTR(y);
   hipLaunchKernelGGL(f32_combine_bwd_kernel, dim3((unsigned)R), dim3(256), 0, (hipStream_t)stream, dy, y, gates,
                      pos_to_row, (int)T, (int)H, (int)k, dyp, dgates);

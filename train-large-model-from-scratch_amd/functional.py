@@ -565,6 +565,64 @@ class _ExpertsRows(torch.autograd.Function):
         return drows, None, dw1, dw3, dw2, None
 
 
+class _ExpertsRowsF32(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, rows, ids, w1, w3, w2):
+        R, H = rows.shape
+        E = w1.shape[0]
+        rows, w1, w3, w2 = _dense(rows), _dense(w1), _dense(w3), _dense(w2)
+        ids32 = _dense(ids.to(torch.int32))
+        counts, offs, pos_to_row, row_to_pos, bad = ops.histogram_scan(ids32, E, return_bad=True)
+        xp = ops.f32_gather_rows(rows, pos_to_row, 1)
+        g = ops.f32_gemm_rows(xp, w1, offs, True)
+        u = ops.f32_gemm_rows(xp, w3, offs, True)
+        act = ops.f32_swiglu(g, u)
+        y = ops.f32_gemm_rows(act, w2, offs, True)
+        out = ops.f32_combine_fwd(y, None, row_to_pos, R, 1)
+        if any(ctx.needs_input_grad):
+            ctx.save_for_backward(xp, g, u, act, offs, pos_to_row, row_to_pos, w1, w3, w2)
+        ctx.mark_non_differentiable(counts, offs, pos_to_row, row_to_pos, bad)
+        ctx.set_materialize_grads(False)
+        ctx.out_shape = out.shape
+        return out, counts, offs, pos_to_row, row_to_pos, bad
+
+    @staticmethod
+    def backward(ctx, dout, *unused):
+        xp, g, u, act, offs, pos_to_row, row_to_pos, w1, w3, w2 = ctx.saved_tensors
+        if dout is None:
+            dout = torch.zeros(ctx.out_shape, dtype=torch.float32, device=xp.device)
+        R, E = dout.shape[0], w1.shape[0]
+        need = ctx.needs_input_grad
+        dyp, _ = ops.f32_combine_bwd(_dense(dout.float()), None, None, pos_to_row, 1)
+        dg, du = ops.f32_swiglu_bwd(ops.f32_gemm_rows(dyp, w2, offs, False), g, u)
+        drows = None
+        if need[0]:
+            dxp = ops.f32_gemm_rows(dg, w1, offs, False)
+            ops.f32_gemm_rows(du, w3, offs, False, out=dxp)
+            drows = ops.f32_permute_bwd(dxp, row_to_pos, R, 1)
+        dw1 = ops.f32_gemm_wgrad(dg, xp, offs, E) if need[2] else None
+        dw3 = ops.f32_gemm_wgrad(du, xp, offs, E) if need[3] else None
+        dw2 = ops.f32_gemm_wgrad(dyp, act, offs, E) if need[4] else None
+        return drows, None, dw1, dw3, dw2
+
+
+def experts_rows_f32(rows: torch.Tensor, ids: torch.Tensor, w1, w3, w2, return_routing: bool = False,
+                     check_ids: bool = False):
+    """`experts_rows` with every tensor and every product in fp32 (rows and weights fp32)."""
+    for name, t in (("rows", rows), ("w1", w1), ("w3", w3), ("w2", w2)):
+        if t.dtype != torch.float32:
+            raise TypeError(f"experts_rows_f32: {name} must be fp32, got {t.dtype}")
+    out, counts, offs, pos_to_row, row_to_pos, bad = _ExpertsRowsF32.apply(rows, ids, w1, w3, w2)
+    if check_ids:
+        n = int(bad.item())
+        if n:
+            raise ValueError(f"experts_rows_f32: {n} of {ids.numel()} expert ids lie outside [0, {w1.shape[0]})")
+    if return_routing:
+        return out, {"counts": counts, "offs": offs, "pos_to_row": pos_to_row, "row_to_pos": row_to_pos,
+                     "bad_ids": bad}
+    return out
+
+
 def experts_rows(rows: torch.Tensor, ids: torch.Tensor, w1, w3, w2, return_routing: bool = False,
                  accumulate_into_grad: bool = False, check_ids: bool = False):
     """One rank's local expert share: rows [R,H] already dispatched to this rank, ids [R]

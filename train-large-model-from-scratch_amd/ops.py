@@ -396,7 +396,8 @@ def f32_gather_rows(x: torch.Tensor, pos_to_row: torch.Tensor, k: int) -> torch.
     return xp
 
 
-def f32_combine_fwd(y: torch.Tensor, gates: torch.Tensor, row_to_pos: torch.Tensor, T: int, k: int):
+def f32_combine_fwd(y: torch.Tensor, gates: torch.Tensor | None, row_to_pos: torch.Tensor, T: int, k: int):
+    """out[t] = sum_j gates[t*k+j] * y[row_to_pos[t*k+j]]; gates None: all ones."""
     _f32(y, gates)
     H = y.shape[-1]
     out = torch.empty(T, H, dtype=torch.float32, device=y.device)
