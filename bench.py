@@ -28,13 +28,13 @@ HBM_PEAK_GBS = 8000.0
 # are in profiles/grouped_gemm_cfg3_pmc.txt.  bench.py cannot run the profiler on itself, so
 # the figures are carried here and refreshed whenever that profile is.
 MEASURED_HBM_BYTES_PER_LAUNCH = {
-    (3, "gemm_gateup_swiglu_fwd_blocked"): 4.019e9,
-    (3, "gemm_gateup_swiglu_fwd"): 4.019e9,
-    (3, "gemm_down_fwd"): 1.849e9,
-    (3, "gemm_dgrad_down_swiglu_bwd_blocked"): 2.452e9,
-    (3, "gemm_dgrad_down_swiglu_bwd"): 2.452e9,
-    (3, "gemm_dgrad_gateup_packed"): 3.760e9,
-    (3, "gemm_dgrad_gateup"): 3.760e9,
+    (3, "gemm_gateup_swiglu_fwd_blocked"): 3.994e9,
+    (3, "gemm_gateup_swiglu_fwd"): 3.994e9,
+    (3, "gemm_down_fwd"): 1.860e9,
+    (3, "gemm_dgrad_down_swiglu_bwd_blocked"): 2.460e9,
+    (3, "gemm_dgrad_down_swiglu_bwd"): 2.460e9,
+    (3, "gemm_dgrad_gateup_packed"): 3.763e9,
+    (3, "gemm_dgrad_gateup"): 3.763e9,
     (3, "gemm_wgrad_down"): 1.074e9,
     (3, "gemm_wgrad"): 1.074e9,
     (3, "gemm_wgrad_pair"): 2.18e9,                # from the average over both weight-gradient launches
@@ -480,6 +480,9 @@ def main():
                          "dense reference (a profiler then sees the launches of the steps only)")
     ap.add_argument("--no-others", action="store_true",
                     help="skip the short runs of the other benchmark configurations (field other_configs)")
+    ap.add_argument("--fp32", action="store_true",
+                    help="time only configuration 3 in fp32 from end to end (the other_configs entry "
+                         "`moe_ffn_f32`) and print its record")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (one rank's share of the MoE layer, "
@@ -497,6 +500,10 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
+    if args.fp32:
+        print(json.dumps(fp32_config3(P, torch, dev, steps=min(args.steps, 5), warmup=min(args.warmup, 2))),
+              flush=True)
+        return 0
     if args.config == 5:
         print(json.dumps(bench_block(args, torch, P, dev, cpu=not args.no_cpu)), flush=True)
         return 0
