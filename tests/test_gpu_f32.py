@@ -288,3 +288,21 @@ def test_f32_rows_entry_matches_the_oracle_in_fp64(P):
         P.experts_rows_f32(rows.cuda(), bad.cuda(), w1.cuda(), w3.cuda(), w2.cuda(), check_ids=True)
     with pytest.raises(TypeError):
         P.experts_rows_f32(rows.cuda().bfloat16(), ids.cuda(), w1.cuda(), w3.cuda(), w2.cuda())
+
+
+def test_f32_layer_is_reproducible_bit_for_bit(P):
+    """Two runs of the fp32 layer on the same inputs give the same bits in every output and
+    gradient (fixed summation orders, no floating-point atomics)."""
+    x, wr, w1, w3, w2, dy, _ = _layer_case(P, 900, 256, 128, 16, 4, seed=77)
+
+    def run():
+        xd = x.cuda().requires_grad_(True)
+        ws = [w.cuda().requires_grad_(True) for w in (w1, w3, w2)]
+        lg = F.linear(x.cuda(), wr.cuda()).requires_grad_(True)
+        out = P.moe_ffn_f32(xd, lg, *ws, 4)
+        out.backward(dy.cuda())
+        return [out.detach(), xd.grad, lg.grad] + [w.grad for w in ws]
+
+    a, b = run(), run()
+    for i, (p, q) in enumerate(zip(a, b)):
+        assert torch.equal(p, q), i
