@@ -355,6 +355,10 @@ int moe_f32_gemm_rows(const float* a, const float* b, const int32_t* offs, int64
  * Experts without rows get exact zeros (are left untouched when accumulating). */
 int moe_f32_gemm_wgrad(const float* a, const float* b, const int32_t* offs, int64_t E, int64_t R,
                        int64_t M, int64_t N, float* dw, int accumulate, void* stream);
+/* Test hook (no counterpart in the reference): the two fp32 GEMM entries choose 64 x 64 or
+ * 128 x 128 output tiles from the shapes; 64 or 128 forces one, 0 restores the choice.  Returns
+ * the previous setting.  Process-wide, not synchronised. */
+int moe_f32_gemm_force_tile(int t);
 
 #ifdef __cplusplus
 }

@@ -54,8 +54,18 @@ def _offsets(counts):
     ([300, 7, 0, 513, 64, 1, 0, 200], 516, 260),
     ([0, 0, 0], 64, 64),                   # no rows at all
 ])
-def test_f32_gemm_rows_and_wgrad(P, counts, N, K):
-    _say("f32 gemm", counts, N, K)
+@pytest.mark.parametrize("tile", [64, 128])
+def test_f32_gemm_rows_and_wgrad(P, counts, N, K, tile):
+    """Both tile sizes on every shape (a launch chooses one from its sizes; the hook forces it)."""
+    _say("f32 gemm", counts, N, K, "tile", tile)
+    before = P.lib.load().cdll.moe_f32_gemm_force_tile(tile)
+    try:
+        _gemm_case(P, counts, N, K)
+    finally:
+        P.lib.load().cdll.moe_f32_gemm_force_tile(before)
+
+
+def _gemm_case(P, counts, N, K):
     ops = P.ops
     E, R = len(counts), int(sum(counts))
     offs = _offsets(counts)

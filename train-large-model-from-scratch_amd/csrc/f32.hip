@@ -3,14 +3,22 @@
 // (model/modules/mlp.py:133-169 with fp32 operands), and so does this file.  Same routing and
 // dispatch kernels as the bf16 path; what differs is the row type of the expert-contiguous
 // buffers (fp32 [R,H] / [R,I]) and the matrix instruction (v_mfma_f32_32x32x2_f32, fp32
-// operands, fp32 accumulate).  A compatibility mode: correct and bounds-checked, 64 x 64 tiles,
-// not tuned towards the fp32 matrix peak.
+// operands, fp32 accumulate).  A compatibility mode: correct and bounds-checked, 64 x 64 or
+// 128 x 128 tiles from plain HIP, 60 to 80 % of the fp32 matrix peak on large shapes.
 #include "common.h"
 
 namespace {
 
-constexpr int TM = 64, TN = 64, TK = 16;
-constexpr int LD = TM + 4;  // floats per LDS row (k-major tiles: row = k, 64 m or n values + pad)
+constexpr int TK = 16;  // depth of a k-tile
+
+// Output tiles of T x T (T = 64 or 128) per workgroup of four waves (2 x 2, each T/2 x T/2 as
+// NB x NB blocks of 32 x 32).  LDS tiles are k-major: row = k, T values of m (or n) + 4 of padding.
+template <int T>
+struct Shape {
+  static constexpr int LD = T + 4;
+  static constexpr int NB = T / 64;   // 32 x 32 blocks per wave and dimension
+  static constexpr int PER = T / 64;  // 16-byte loads per thread, operand and k-tile
+};
 
 struct F32Gemm {
   const float* A;
@@ -22,67 +30,116 @@ struct F32Gemm {
   int accumulate;
 };
 
-// 64 x 16 tile of an operand whose k index is contiguous in memory (element (i, k) at
-// base[i * ld + k]): thread t takes row t/4 and the four k values 4*(t%4).., and writes them
-// transposed into the k-major LDS tile.
-__device__ __forceinline__ f32x4 load_kcont(const float* base, long long ld, int i0, int i_lim, int k0, int K) {
-  const int i = i0 + (threadIdx.x >> 2), k = k0 + (threadIdx.x & 3) * 4;
-  f32x4 v = {0.f, 0.f, 0.f, 0.f};
-  if (i < i_lim && k < K) v = *reinterpret_cast<const f32x4*>(base + (long long)i * ld + k);  // (K % 4 == 0)
-  return v;
-}
-__device__ __forceinline__ void stage_kcont(float* s, f32x4 v) {
-  const int i = threadIdx.x >> 2, k = (threadIdx.x & 3) * 4;
+// T x 16 tile of an operand whose k index is contiguous in memory (element (i, k) at
+// base[i * ld + k]): thread t takes rows t/4 (+64) and the four k values 4*(t%4).., and writes
+// them transposed into the k-major LDS tile.
+template <int T>
+__device__ __forceinline__ void load_kcont(f32x4 (&v)[Shape<T>::PER], const float* base, long long ld, int i0,
+                                           int i_lim, int k0, int K) {
+  const int k = k0 + (threadIdx.x & 3) * 4;
 #pragma unroll
-  for (int x = 0; x < 4; ++x) s[(k + x) * LD + i] = v[x];
+  for (int r = 0; r < Shape<T>::PER; ++r) {
+    const int i = i0 + (threadIdx.x >> 2) + 64 * r;
+    v[r] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (i < i_lim && k < K) v[r] = *reinterpret_cast<const f32x4*>(base + (long long)i * ld + k);  // (K % 4 == 0)
+  }
 }
-// 16 x 64 tile of an operand whose m (or n) index is contiguous (element (k, i) at
-// base[k * ld + i]): thread t takes k row t/16 and the four values 4*(t%16)..
-__device__ __forceinline__ f32x4 load_icont(const float* base, long long ld, int k0, int k_lim, int i0, int i_lim) {
-  const int k = k0 + (threadIdx.x >> 4), i = i0 + (threadIdx.x & 15) * 4;
-  f32x4 v = {0.f, 0.f, 0.f, 0.f};
-  if (k < k_lim && i < i_lim) v = *reinterpret_cast<const f32x4*>(base + (long long)k * ld + i);  // (i_lim % 4 == 0)
-  return v;
+template <int T>
+__device__ __forceinline__ void stage_kcont(float* s, const f32x4 (&v)[Shape<T>::PER]) {
+  const int k = (threadIdx.x & 3) * 4;
+#pragma unroll
+  for (int r = 0; r < Shape<T>::PER; ++r) {
+    const int i = (threadIdx.x >> 2) + 64 * r;
+#pragma unroll
+    for (int x = 0; x < 4; ++x) s[(k + x) * Shape<T>::LD + i] = v[r][x];
+  }
 }
-__device__ __forceinline__ void stage_icont(float* s, f32x4 v) {
-  *reinterpret_cast<f32x4*>(s + (threadIdx.x >> 4) * LD + (threadIdx.x & 15) * 4) = v;
+// 16 x T tile of an operand whose m (or n) index is contiguous (element (k, i) at
+// base[k * ld + i]): T/4 threads per k row take four values each, 1024/T k rows per pass.
+template <int T>
+__device__ __forceinline__ void load_icont(f32x4 (&v)[Shape<T>::PER], const float* base, long long ld, int k0,
+                                           int k_lim, int i0, int i_lim) {
+  const int i = i0 + (threadIdx.x % (T / 4)) * 4;
+#pragma unroll
+  for (int r = 0; r < Shape<T>::PER; ++r) {
+    const int k = k0 + threadIdx.x / (T / 4) + (1024 / T) * r;
+    v[r] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (k < k_lim && i < i_lim) v[r] = *reinterpret_cast<const f32x4*>(base + (long long)k * ld + i);  // (i_lim % 4 == 0)
+  }
+}
+template <int T>
+__device__ __forceinline__ void stage_icont(float* s, const f32x4 (&v)[Shape<T>::PER]) {
+#pragma unroll
+  for (int r = 0; r < Shape<T>::PER; ++r)
+    *reinterpret_cast<f32x4*>(s + (threadIdx.x / (T / 4) + (1024 / T) * r) * Shape<T>::LD +
+                              (threadIdx.x % (T / 4)) * 4) = v[r];
 }
 
-// One k-tile of 16 from LDS: wave (wm, wn) of the 2 x 2 owns a 32 x 32 block.  The operands go
-// in swapped, so that a lane ends up with row lane%32 of the block and four consecutive
-// columns per group of four accumulator registers (columns 8g + 4*(lane/32) .. +3).
-__device__ __forceinline__ void mma_tile(const float* sA, const float* sB, int wm, int wn, f32x16& acc) {
+// One k-tile of 16 from LDS.  The operands go in swapped, so that a lane ends up with row
+// lane%32 of a 32 x 32 block and four consecutive columns per group of four accumulator
+// registers (columns 8g + 4*(lane/32) .. +3).
+template <int T>
+__device__ __forceinline__ void mma_tile(const float* sA, const float* sB, int wm, int wn,
+                                         f32x16 (&acc)[Shape<T>::NB][Shape<T>::NB]) {
+  constexpr int NB = Shape<T>::NB, LD = Shape<T>::LD;
   const int l32 = threadIdx.x & 31, lh = (threadIdx.x >> 5) & 1;
 #pragma unroll
   for (int kk = 0; kk < TK / 2; ++kk) {
-    const float a = sA[(2 * kk + lh) * LD + wm * 32 + l32];
-    const float b = sB[(2 * kk + lh) * LD + wn * 32 + l32];
-    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(b, a, acc, 0, 0, 0);
+    float a[NB], b[NB];
+#pragma unroll
+    for (int x = 0; x < NB; ++x) {
+      a[x] = sA[(2 * kk + lh) * LD + (wm * NB + x) * 32 + l32];
+      b[x] = sB[(2 * kk + lh) * LD + (wn * NB + x) * 32 + l32];
+    }
+#pragma unroll
+    for (int bi = 0; bi < NB; ++bi)
+#pragma unroll
+      for (int bj = 0; bj < NB; ++bj)
+        acc[bi][bj] = __builtin_amdgcn_mfma_f32_32x32x2f32(b[bj], a[bi], acc[bi][bj], 0, 0, 0);
   }
 }
 
-__device__ __forceinline__ void store_block(float* C, long long ldc, int m0, int m_lim, int n0, int n_lim,
-                                            int wm, int wn, const f32x16& acc, bool accumulate) {
+template <int T>
+__device__ __forceinline__ void store_tile(float* C, long long ldc, int m0, int m_lim, int n0, int n_lim, int wm,
+                                           int wn, const f32x16 (&acc)[Shape<T>::NB][Shape<T>::NB],
+                                           bool accumulate) {
+  constexpr int NB = Shape<T>::NB;
   const int l32 = threadIdx.x & 31, lh = (threadIdx.x >> 5) & 1;
-  const int m = m0 + wm * 32 + l32;
-  if (m >= m_lim) return;
 #pragma unroll
-  for (int g = 0; g < 4; ++g) {
-    const int n = n0 + wn * 32 + 8 * g + 4 * lh;
-    if (n >= n_lim) continue;  // (n_lim % 4 == 0: the four columns are inside or outside together)
-    f32x4* dst = reinterpret_cast<f32x4*>(C + (long long)m * ldc + n);
-    f32x4 v = {acc[4 * g], acc[4 * g + 1], acc[4 * g + 2], acc[4 * g + 3]};
-    if (accumulate) v += *dst;
-    *dst = v;
+  for (int bi = 0; bi < NB; ++bi) {
+    const int m = m0 + (wm * NB + bi) * 32 + l32;
+    if (m >= m_lim) continue;
+#pragma unroll
+    for (int bj = 0; bj < NB; ++bj)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int n = n0 + (wn * NB + bj) * 32 + 8 * g + 4 * lh;
+        if (n >= n_lim) continue;  // (n_lim % 4 == 0: the four columns are inside or outside together)
+        f32x4* dst = reinterpret_cast<f32x4*>(C + (long long)m * ldc + n);
+        f32x4 v = {acc[bi][bj][4 * g], acc[bi][bj][4 * g + 1], acc[bi][bj][4 * g + 2], acc[bi][bj][4 * g + 3]};
+        if (accumulate) v += *dst;
+        *dst = v;
+      }
   }
+}
+
+template <int T>
+__device__ __forceinline__ void clear(f32x16 (&acc)[Shape<T>::NB][Shape<T>::NB]) {
+#pragma unroll
+  for (int bi = 0; bi < Shape<T>::NB; ++bi)
+#pragma unroll
+    for (int bj = 0; bj < Shape<T>::NB; ++bj)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[bi][bj][i] = 0.f;
 }
 
 // Row-ragged: C[r, :] (+)= A[r, :] x B_e for the rows r of expert e.  A [R,K] row-major;
 // B_e = B + e*N*K holds either [N,K] (B_KCONT: C = A B_e^T, the forward products) or [K,N]
-// (C = A B_e, the input gradients).  blockIdx.x counts 64-row tiles over all experts (an
-// expert's last tile may be short), blockIdx.y 64-column tiles.
-template <bool B_KCONT>
+// (C = A B_e, the input gradients).  blockIdx.x counts T-row tiles over all experts (an
+// expert's last tile may be short), blockIdx.y T-column tiles.
+template <int T, bool B_KCONT>
 __global__ __launch_bounds__(256) void f32_gemm_rows_kernel(F32Gemm p) {
+  constexpr int LD = Shape<T>::LD, PER = Shape<T>::PER, NB = Shape<T>::NB;
   __shared__ __align__(16) float sA[TK * LD], sB[TK * LD];
   __shared__ int s_tile[3];
   if (threadIdx.x == 0) {
@@ -90,10 +147,10 @@ __global__ __launch_bounds__(256) void f32_gemm_rows_kernel(F32Gemm p) {
     for (int e = 0; e < p.E; ++e) {
       const int b = p.offs[e], n = p.offs[e + 1] - b;
       if (n <= 0 || b < 0 || b + n > p.R) continue;  // (empty, or offsets no dispatch would produce)
-      const int nt = (n + TM - 1) / TM;
+      const int nt = (n + T - 1) / T;
       if ((int)blockIdx.x < seen + nt) {
         found = e;
-        row0 = b + ((int)blockIdx.x - seen) * TM;
+        row0 = b + ((int)blockIdx.x - seen) * T;
         row_end = b + n;
         break;
       }
@@ -105,59 +162,78 @@ __global__ __launch_bounds__(256) void f32_gemm_rows_kernel(F32Gemm p) {
   }
   __syncthreads();
   const int e = s_tile[0], row0 = s_tile[1], row_end = s_tile[2];
-  if (e < 0) return;  // (the grid is sized for the worst case: R/64 + E tiles)
-  const int n0 = blockIdx.y * TN;
+  if (e < 0) return;  // (the grid is sized for the worst case: R/T + E tiles)
+  const int n0 = blockIdx.y * T;
   const float* Be = p.B + (long long)e * p.N * p.K;
   const int wv = threadIdx.x >> 6, wm = wv >> 1, wn = wv & 1;
-  f32x16 acc;
-#pragma unroll
-  for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-  auto fetch_b = [&](int k0) {
-    if constexpr (B_KCONT) return load_kcont(Be, p.K, n0, p.N, k0, p.K);
-    else return load_icont(Be, p.N, k0, p.K, n0, p.N);
+  f32x16 acc[NB][NB];
+  clear<T>(acc);
+  f32x4 ra[PER], rb[PER];
+  auto fetch = [&](int k0) {
+    load_kcont<T>(ra, p.A, p.K, row0, row_end, k0, p.K);
+    if constexpr (B_KCONT) load_kcont<T>(rb, Be, p.K, n0, p.N, k0, p.K);
+    else load_icont<T>(rb, Be, p.N, k0, p.K, n0, p.N);
   };
-  f32x4 ra = load_kcont(p.A, p.K, row0, row_end, 0, p.K), rb = fetch_b(0);
+  fetch(0);
   for (int k0 = 0; k0 < p.K; k0 += TK) {
-    stage_kcont(sA, ra);
-    if constexpr (B_KCONT) stage_kcont(sB, rb);
-    else stage_icont(sB, rb);
+    stage_kcont<T>(sA, ra);
+    if constexpr (B_KCONT) stage_kcont<T>(sB, rb);
+    else stage_icont<T>(sB, rb);
     __syncthreads();
-    if (k0 + TK < p.K) {
-      ra = load_kcont(p.A, p.K, row0, row_end, k0 + TK, p.K);
-      rb = fetch_b(k0 + TK);
-    }
-    mma_tile(sA, sB, wm, wn, acc);
+    if (k0 + TK < p.K) fetch(k0 + TK);
+    mma_tile<T>(sA, sB, wm, wn, acc);
     __syncthreads();
   }
-  store_block(p.C, p.N, row0, row_end, n0, p.N, wm, wn, acc, p.accumulate != 0);
+  store_tile<T>(p.C, p.N, row0, row_end, n0, p.N, wm, wn, acc, p.accumulate != 0);
 }
 
 // k-ragged: C_e[m, n] (+)= sum over the rows r of expert e of A[r, m] * B[r, n]  (the weight
 // gradients).  A [R,M], B [R,N] row-major, C [E,M,N].  grid = (N tiles, M tiles, E).  An expert
 // without rows gets zeros (or is left alone when accumulating).
+template <int T>
 __global__ __launch_bounds__(256) void f32_gemm_wgrad_kernel(F32Gemm p) {
+  constexpr int LD = Shape<T>::LD, PER = Shape<T>::PER, NB = Shape<T>::NB;
   __shared__ __align__(16) float sA[TK * LD], sB[TK * LD];
-  const int e = blockIdx.z, n0 = blockIdx.x * TN, m0 = blockIdx.y * TM;
+  const int e = blockIdx.z, n0 = blockIdx.x * T, m0 = blockIdx.y * T;
   int b = p.offs[e], end = p.offs[e + 1];
   if (b < 0 || end > p.R || end < b) b = end = 0;
   const int wv = threadIdx.x >> 6, wm = wv >> 1, wn = wv & 1;
-  f32x16 acc;
-#pragma unroll
-  for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-  f32x4 ra = load_icont(p.A, p.M, b, end, m0, p.M), rb = load_icont(p.B, p.N, b, end, n0, p.N);
+  f32x16 acc[NB][NB];
+  clear<T>(acc);
+  f32x4 ra[PER], rb[PER];
+  load_icont<T>(ra, p.A, p.M, b, end, m0, p.M);
+  load_icont<T>(rb, p.B, p.N, b, end, n0, p.N);
   for (int k0 = b; k0 < end; k0 += TK) {
-    stage_icont(sA, ra);
-    stage_icont(sB, rb);
+    stage_icont<T>(sA, ra);
+    stage_icont<T>(sB, rb);
     __syncthreads();
     if (k0 + TK < end) {
-      ra = load_icont(p.A, p.M, k0 + TK, end, m0, p.M);
-      rb = load_icont(p.B, p.N, k0 + TK, end, n0, p.N);
+      load_icont<T>(ra, p.A, p.M, k0 + TK, end, m0, p.M);
+      load_icont<T>(rb, p.B, p.N, k0 + TK, end, n0, p.N);
     }
-    mma_tile(sA, sB, wm, wn, acc);
+    mma_tile<T>(sA, sB, wm, wn, acc);
     __syncthreads();
   }
   if (end == b && p.accumulate) return;
-  store_block(p.C + (long long)e * p.M * p.N, p.N, m0, p.M, n0, p.N, wm, wn, acc, p.accumulate != 0);
+  store_tile<T>(p.C + (long long)e * p.M * p.N, p.N, m0, p.M, n0, p.N, wm, wn, acc, p.accumulate != 0);
+}
+
+// The larger tile halves the operand traffic per flop; a launch takes it when it still gives
+// every compute unit at least two tiles.
+int f32_forced_tile = 0;
+int f32_units[MOE_MAX_DEVICES];
+int f32_compute_units() {
+  const int dev = moe_current_device();
+  if (f32_units[dev] <= 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    f32_units[dev] = n;
+  }
+  return f32_units[dev];
+}
+bool f32_large_tiles(int64_t tiles128) {
+  if (f32_forced_tile) return f32_forced_tile == 128;
+  return tiles128 >= 2 * (int64_t)f32_compute_units();
 }
 
 // ---- row movers and element-wise kernels (one workgroup per row, 16-byte accesses)
@@ -388,9 +464,16 @@ extern "C" int moe_f32_gemm_rows(const float* a, const float* b, const int32_t* 
   MOE_CHECK_PTR(c);
   if (!offs) return MOE_ERR_NULL;
   F32Gemm p{a, b, c, offs, (int)E, (int)R, 0, (int)N, (int)K, accumulate};
-  const dim3 grid((unsigned)(R / TM + E), (unsigned)((N + TN - 1) / TN));
-  if (b_k_contiguous) hipLaunchKernelGGL(f32_gemm_rows_kernel<true>, grid, dim3(256), 0, (hipStream_t)stream, p);
-  else hipLaunchKernelGGL(f32_gemm_rows_kernel<false>, grid, dim3(256), 0, (hipStream_t)stream, p);
+  hipStream_t s = (hipStream_t)stream;
+  if (f32_large_tiles((R / 128 + E) * ((N + 127) / 128))) {
+    const dim3 grid((unsigned)(R / 128 + E), (unsigned)((N + 127) / 128));
+    if (b_k_contiguous) hipLaunchKernelGGL((f32_gemm_rows_kernel<128, true>), grid, dim3(256), 0, s, p);
+    else hipLaunchKernelGGL((f32_gemm_rows_kernel<128, false>), grid, dim3(256), 0, s, p);
+  } else {
+    const dim3 grid((unsigned)(R / 64 + E), (unsigned)((N + 63) / 64));
+    if (b_k_contiguous) hipLaunchKernelGGL((f32_gemm_rows_kernel<64, true>), grid, dim3(256), 0, s, p);
+    else hipLaunchKernelGGL((f32_gemm_rows_kernel<64, false>), grid, dim3(256), 0, s, p);
+  }
   return moe_launch_status();
 }
 
@@ -407,7 +490,21 @@ extern "C" int moe_f32_gemm_wgrad(const float* a, const float* b, const int32_t*
     MOE_CHECK_PTR(b);
   }
   F32Gemm p{a, b, dw, offs, (int)E, (int)R, (int)M, (int)N, 0, accumulate};
-  const dim3 grid((unsigned)((N + TN - 1) / TN), (unsigned)((M + TM - 1) / TM), (unsigned)E);
-  hipLaunchKernelGGL(f32_gemm_wgrad_kernel, grid, dim3(256), 0, (hipStream_t)stream, p);
+  if (f32_large_tiles(E * ((M + 127) / 128) * ((N + 127) / 128))) {
+    const dim3 grid((unsigned)((N + 127) / 128), (unsigned)((M + 127) / 128), (unsigned)E);
+    hipLaunchKernelGGL(f32_gemm_wgrad_kernel<128>, grid, dim3(256), 0, (hipStream_t)stream, p);
+  } else {
+    const dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64), (unsigned)E);
+    hipLaunchKernelGGL(f32_gemm_wgrad_kernel<64>, grid, dim3(256), 0, (hipStream_t)stream, p);
+  }
   return moe_launch_status();
+}
+
+// Test hook: 0 lets every fp32 GEMM launch choose its tile (the default), 64 or 128 forces it.
+// Process-wide and not synchronised: for tests, not for production callers.  Returns the previous
+// setting.
+extern "C" int moe_f32_gemm_force_tile(int t) {
+  const int before = f32_forced_tile;
+  if (t == 0 || t == 64 || t == 128) f32_forced_tile = t;
+  return before;
 }

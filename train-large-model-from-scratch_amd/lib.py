@@ -66,6 +66,7 @@ SIGNATURES = {
     "moe_f32_swiglu_bwd": (_int, [_vp, _vp, _vp, _i64, _vp, _vp, _vp]),
     "moe_f32_gemm_rows": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp, _int, _vp]),
     "moe_f32_gemm_wgrad": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _int, _vp]),
+    "moe_f32_gemm_force_tile": (_int, [_int]),
 }
 
 ERRORS = {-1: "MOE_ERR_NULL", -2: "MOE_ERR_SHAPE", -3: "MOE_ERR_LIMIT", -4: "MOE_ERR_DTYPE",
