@@ -102,3 +102,33 @@ def test_compiled_with_the_inductor_backend(pkg, lib):
         assert rel < 1e-2, (n, rel)
         if same_logits and n in ("out", "experts_gate_weights", "experts_up_weights", "experts_down_weights"):
             assert torch.equal(a, b), n
+
+
+def test_compiled_fp32_call_takes_the_fp32_operators(pkg, lib):
+    """fp32 parameters and input, no autocast: the compiled module stays one graph, runs the
+    fp32 pair of operators and gives the bits of the eager fp32 call (same kernels, same order;
+    the router product is the module's own nn.Linear in both)."""
+    traced = importlib.import_module(pkg.__name__ + ".traced")
+    m, x, dy = _case(pkg, torch.float32)
+    x2 = x.reshape(-1, 256).requires_grad_(True)
+    logits = torch.nn.functional.linear(x2.detach(), m.router.weight.detach()).requires_grad_(True)
+    args = (x2, logits, m.experts_gate_weights, m.experts_up_weights, m.experts_down_weights, 2, True)
+    torch.library.opcheck(traced.ffn_f32_fwd, args,
+                          test_utils=("test_schema", "test_faketensor", "test_autograd_registration"))
+
+    def run(mod):
+        m.zero_grad(set_to_none=True)
+        xi = x.clone().requires_grad_(True)
+        out, lg = mod(xi)
+        out.backward(dy)
+        return [out.detach(), lg.detach(), xi.grad] + [p.grad.clone() for p in m.parameters()]
+
+    eager = run(m)
+    compiled = run(torch.compile(m, backend="aot_eager", fullgraph=True))
+    names = ["out", "gate_logits", "dx"] + [n for n, _ in m.named_parameters()]
+    for n, a, b in zip(names, eager, compiled):
+        assert a.dtype == torch.float32 and b.dtype == torch.float32 and a.shape == b.shape, n
+        rel = ((a - b).norm() / a.norm().clamp_min(1e-30)).item()
+        _say(f"  {n}: rel diff compiled vs eager {rel:.2e}")
+        assert rel < 1e-5, (n, rel)
+    assert torch.equal(eager[0], compiled[0])

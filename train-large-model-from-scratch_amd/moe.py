@@ -181,16 +181,18 @@ class MoE(nn.Module):
         return all(w.dtype == torch.float32 for w in (self.router.weight, self.experts_gate_weights,
                                                       self.experts_up_weights, self.experts_down_weights))
 
+    @staticmethod
     @torch._dynamo.disable
-    def _experts_f32(self, x2d: torch.Tensor, logits2d: torch.Tensor) -> torch.Tensor:
-        return moe_ffn_f32(x2d, logits2d, self.experts_gate_weights, self.experts_up_weights,
-                           self.experts_down_weights, self.top_k)
+    def _experts_f32(x2d, logits2d, w1, w3, w2, k) -> torch.Tensor:
+        return moe_ffn_f32(x2d, logits2d, w1, w3, w2, k)
 
     def forward(self, x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
         B, T, D = x.size()
-        if not torch.compiler.is_compiling() and self._runs_in_fp32(x):
+        if self._runs_in_fp32(x):
             gate_logits = self.router(x)  # fp32 product and fp32 gradients, as nn.Linear gives them
-            out = self._experts_f32(x.reshape(B * T, D), gate_logits.reshape(B * T, self.num_experts))
+            ffn = traced.moe_ffn_f32 if torch.compiler.is_compiling() else self._experts_f32
+            out = ffn(x.reshape(B * T, D), gate_logits.reshape(B * T, self.num_experts),
+                      self.experts_gate_weights, self.experts_up_weights, self.experts_down_weights, self.top_k)
             return out.reshape(B, T, D), gate_logits
         if torch.compiler.is_compiling():
             # under torch.compile (trainer.py:130-131): the same kernels as registered

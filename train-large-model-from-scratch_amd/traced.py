@@ -9,7 +9,10 @@ can keep `MoE.forward` inside one graph, forward and backward: the kernels stay 
 everything around them is traced.  `MoE.forward` takes this route only while it is being
 traced; eager calls use `functional.moe_ffn` (same kernels, plus the cached weight copies).
 
-Semantics are those of `functional.moe_ffn`: bf16 matrix-core compute with fp32
+A second pair, `moe_gfx950::ffn_f32_fwd` / `ffn_f32_bwd` at the end of the file, does the same
+for the fp32 path (`functional.moe_ffn_f32`).
+
+Semantics of the first pair are those of `functional.moe_ffn`: bf16 matrix-core compute with fp32
 accumulation, output and input gradient in the dtype of x, weight gradients in the dtype of
 the weights.  fp32 weights are rounded to bf16 inside the forward operator (three casts per
 call, what the reference pays too, mlp.py:154-157 under autocast) and the copies are handed to
@@ -130,3 +133,94 @@ def moe_ffn(x: Tensor, logits: Tensor, w1: Tensor, w3: Tensor, w2: Tensor, k: in
     """Traceable counterpart of `functional.moe_ffn(x, logits, w1, w3, w2, k)`."""
     train = torch.is_grad_enabled() and any(t.requires_grad for t in (x, logits, w1, w3, w2))
     return ffn_fwd(x, logits, w1, w3, w2, k, train)[0]
+
+
+# ---- the same pair of operators for the fp32 path (functional.moe_ffn_f32) ------------------------
+
+@torch.library.custom_op("moe_gfx950::ffn_f32_fwd", mutates_args=(), device_types="cuda")
+def ffn_f32_fwd(x: Tensor, logits: Tensor, w1: Tensor, w3: Tensor, w2: Tensor, k: int,
+                train: bool) -> tuple[Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor,
+                                      Tensor, Tensor, Tensor]:
+    """-> out, ids, gates, offs, pos_to_row, row_to_pos, xp, g, u, act, y (all floating point
+    tensors fp32).  Without `train` xp, g, u, act and y are empty."""
+    T, H = x.shape
+    E = logits.shape[1]
+    x, logits = ops.dense(x), ops.dense(logits)
+    w1, w3, w2 = ops.dense(w1), ops.dense(w3), ops.dense(w2)
+    ids, gates = ops.router_topk(logits, k, None)
+    _, offs, pos_to_row, row_to_pos = ops.histogram_scan(ids, E)
+    xp = ops.f32_gather_rows(x, pos_to_row, k)
+    g = ops.f32_gemm_rows(xp, w1, offs, True)
+    u = ops.f32_gemm_rows(xp, w3, offs, True)
+    act = ops.f32_swiglu(g, u)
+    y = ops.f32_gemm_rows(act, w2, offs, True)
+    out = ops.f32_combine_fwd(y, gates, row_to_pos, T, k)
+    if not train:
+        e = _empty(x, torch.float32)
+        xp, g, u, act, y = e, e.clone(), e.clone(), e.clone(), e.clone()
+    return out, ids, gates, offs, pos_to_row, row_to_pos, xp, g, u, act, y
+
+
+@ffn_f32_fwd.register_fake
+def _(x, logits, w1, w3, w2, k, train):
+    T, H = x.shape
+    E, I = logits.shape[1], w1.shape[1]
+    R = T * k
+    i32 = lambda *s: x.new_empty(s, dtype=torch.int32)
+    f32 = lambda *s: x.new_empty(s, dtype=torch.float32)
+    rh, ri = ((R, H), (R, I)) if train else ((0,), (0,))
+    return (f32(T, H), i32(R), f32(R), i32(E + 1), i32(R), i32(R), f32(*rh), f32(*ri), f32(*ri), f32(*ri),
+            f32(*rh))
+
+
+@torch.library.custom_op("moe_gfx950::ffn_f32_bwd", mutates_args=(), device_types="cuda")
+def ffn_f32_bwd(dout: Tensor, xp: Tensor, g: Tensor, u: Tensor, act: Tensor, y: Tensor, gates: Tensor,
+                ids: Tensor, offs: Tensor, pos_to_row: Tensor, row_to_pos: Tensor, w1: Tensor, w3: Tensor,
+                w2: Tensor, k: int) -> tuple[Tensor, Tensor, Tensor, Tensor, Tensor]:
+    """-> dx, dlogits, dw1, dw3, dw2 (fp32)."""
+    T = dout.shape[0]
+    E = offs.numel() - 1
+    w1, w3, w2 = ops.dense(w1), ops.dense(w3), ops.dense(w2)
+    dyp, dgates = ops.f32_combine_bwd(ops.dense(dout.float()), y, gates, pos_to_row, k)
+    dg, du = ops.f32_swiglu_bwd(ops.f32_gemm_rows(dyp, w2, offs, False), g, u)
+    dxp = ops.f32_gemm_rows(dg, w1, offs, False)
+    ops.f32_gemm_rows(du, w3, offs, False, out=dxp)
+    dx = ops.f32_permute_bwd(dxp, row_to_pos, T, k)
+    dw1 = ops.f32_gemm_wgrad(dg, xp, offs, E)
+    dw3 = ops.f32_gemm_wgrad(du, xp, offs, E)
+    dw2 = ops.f32_gemm_wgrad(dyp, act, offs, E)
+    dlogits = ops.router_topk_bwd(gates, dgates, ids, T, E, k, torch.float32)
+    return dx, dlogits, dw1, dw3, dw2
+
+
+@ffn_f32_bwd.register_fake
+def _(dout, xp, g, u, act, y, gates, ids, offs, pos_to_row, row_to_pos, w1, w3, w2, k):
+    T, H = dout.shape
+    E = offs.shape[0] - 1
+    f32 = lambda *s: dout.new_empty(s, dtype=torch.float32)
+    return f32(T, H), f32(T, E), f32(*w1.shape), f32(*w3.shape), f32(*w2.shape)
+
+
+def _setup_context_f32(ctx, inputs, output):
+    x, logits, w1, w3, w2, k, train = inputs
+    out, ids, gates, offs, pos_to_row, row_to_pos, xp, g, u, act, y = output
+    ctx.save_for_backward(xp, g, u, act, y, gates, ids, offs, pos_to_row, row_to_pos, w1, w3, w2)
+    ctx.k, ctx.train = k, train
+
+
+def _backward_f32(ctx, dout, *unused):
+    if not ctx.train:
+        raise RuntimeError("moe_gfx950::ffn_f32_fwd was called with train=False: nothing was saved for backward")
+    xp, g, u, act, y, gates, ids, offs, pos_to_row, row_to_pos, w1, w3, w2 = ctx.saved_tensors
+    dx, dlogits, dw1, dw3, dw2 = ffn_f32_bwd(dout, xp, g, u, act, y, gates, ids, offs, pos_to_row, row_to_pos,
+                                             w1, w3, w2, ctx.k)
+    return dx, dlogits, dw1, dw3, dw2, None, None
+
+
+ffn_f32_fwd.register_autograd(_backward_f32, setup_context=_setup_context_f32)
+
+
+def moe_ffn_f32(x: Tensor, logits: Tensor, w1: Tensor, w3: Tensor, w2: Tensor, k: int) -> Tensor:
+    """Traceable counterpart of `functional.moe_ffn_f32(x, logits, w1, w3, w2, k)`."""
+    train = torch.is_grad_enabled() and any(t.requires_grad for t in (x, logits, w1, w3, w2))
+    return ffn_f32_fwd(x, logits, w1, w3, w2, k, train)[0]
