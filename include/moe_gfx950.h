@@ -318,6 +318,19 @@ int moe_rmsnorm_bwd(const void* x, int x_dtype, const float* weight, const float
  * mlp.py:154-157 under trainer.py:209-211). */
 int moe_cast_f32_bf16(const float* src, uint16_t* dst, int64_t n, void* stream);
 
+/* ---- the forward pass in one call ---------------------------------------------------
+ * mlp.py:101-167 for a caller that wants only the output (inference, evaluation, a forward
+ * under no_grad): routing, dispatch, row gather, both grouped GEMMs and the combine enqueued
+ * back to back, every intermediate in `workspace` (moe_ffn_forward_workspace_bytes, 256-byte
+ * aligned pieces; contents unspecified afterwards).  x [T,H] and logits [T,E] bf16 or f32, bias
+ * f32 [E] or NULL, weights bf16 as stored, out [T,H] of out_dtype.  The same kernels in the same
+ * order as the separate entry points: the same bits. */
+int64_t moe_ffn_forward_workspace_bytes(int64_t T, int64_t H, int64_t E, int64_t I, int64_t k);
+int moe_ffn_forward(const void* x, int x_dtype, const void* logits, int logits_dtype,
+                    const float* bias, const uint16_t* w1, const uint16_t* w3, const uint16_t* w2,
+                    int64_t T, int64_t H, int64_t E, int64_t I, int64_t k, void* out, int out_dtype,
+                    void* workspace, int64_t workspace_bytes, void* stream);
+
 /* ---- the path in fp32 ---------------------------------------------------------------
  * For a layer that runs without autocast on fp32 tensors: the reference then keeps every
  * step of mlp.py:104-169 in fp32 (the three bmm's of :154-157 included) and so do these

@@ -914,3 +914,46 @@ def test_two_host_threads_on_two_streams(P):
         assert len(results[i]) == 1
         for a, b in zip(results[i][0], serial[i]):
             assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("x_dtype,k,bias", [(torch.bfloat16, 2, False), (torch.float32, 2, True),
+                                            (torch.bfloat16, 1, False), (torch.float32, 8, False)])
+def test_forward_only_call_gives_the_bits_of_the_differentiable_one(P, x_dtype, k, bias):
+    """With nothing to differentiate (no input requires a gradient, or grad mode is off) the whole
+    forward pass goes to the library as one call (`moe_ffn_forward`): the same kernels in the same
+    order, so `out` and the logits are bit-identical to the call that keeps its intermediates."""
+    T, H, I, E = 777, 256, 128, 8
+    g = torch.Generator().manual_seed(3 + k)
+    x = torch.randn(T, H, generator=g).to(x_dtype).cuda()
+    wr = (torch.randn(E, H, generator=g) * 0.3).to(torch.bfloat16).cuda()
+    w1, w3, w2 = ((torch.randn(*s_, generator=g) * 0.1).to(torch.bfloat16).cuda()
+                  for s_ in ((E, I, H), (E, I, H), (E, H, I)))
+    b = torch.randn(E, generator=g).cuda() if bias else None
+    seen = []
+
+    class Obs:
+        def before(self, name):
+            seen.append(name)
+
+        def after(self, name):
+            pass
+
+    L = P.lib.load()
+    # the differentiable call (x requires a gradient)
+    xg = x.clone().requires_grad_(True)
+    out_g, lg_g = P.routed_moe(xg, wr, w1, w3, w2, k, bias=b)
+    L.observer = Obs()
+    try:
+        out_o, _ = P.routed_moe(x, wr, w1, w3, w2, k, bias=b)   # observed: launch by launch
+    finally:
+        L.observer = None
+    assert "moe_ffn_forward" not in seen and "moe_gemm_down_fwd" in seen
+    out_f, lg_f = P.routed_moe(x, wr, w1, w3, w2, k, bias=b)      # forward only: one call
+    with torch.no_grad():
+        out_n, _ = P.routed_moe(xg, wr, w1, w3, w2, k, bias=b)
+    assert out_f.dtype == x_dtype and torch.equal(out_f, out_g.detach()) and torch.equal(lg_f, lg_g.detach())
+    assert torch.equal(out_n, out_f) and torch.equal(out_o, out_f)
+    # the entry that is handed the logits
+    out_m = P.moe_ffn(x, lg_f, w1, w3, w2, k, bias=b)
+    out_mg = P.moe_ffn(xg, lg_f, w1, w3, w2, k, bias=b)
+    assert torch.equal(out_m, out_mg.detach()) and torch.equal(out_m, out_f)

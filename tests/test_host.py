@@ -167,6 +167,7 @@ _OPTIONAL_POINTERS = {
     "moe_combine_fwd": {"gates"}, "moe_combine_fwd_residual": {"gates"},
     "moe_combine_bwd": {"gates"}, "moe_combine_bwd_by_token": {"gates"},
     "moe_rmsnorm_bwd": {"d2", "dres"},
+    "moe_ffn_forward": {"bias"},
     "moe_f32_combine_fwd": {"gates"}, "moe_f32_combine_bwd": {"y", "gates", "dgates"},
 }
 

@@ -8,7 +8,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 INCLUDE = os.path.join(os.path.dirname(PKG_DIR), "include")
 LIB_PATH = os.path.join(PKG_DIR, "libmoe_gfx950.so")
-SOURCES = ("route.hip", "dispatch.hip", "norm.hip", "gemm.hip", "f32.hip")
+SOURCES = ("route.hip", "dispatch.hip", "norm.hip", "gemm.hip", "f32.hip", "layer.hip")
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",

@@ -292,6 +292,20 @@ class _MoEFFN(torch.autograd.Function):
         return dx, dlogits, dw1, dw3, dw2, None, dbias, None, None
 
 
+def _forward_only(*tensors) -> bool:
+    """Whether a call needs nothing kept for a backward pass: then the whole forward goes to the
+    library as one call (`ops.ffn_forward`).  Not while a launch observer is installed: it wants
+    to see the launches one by one."""
+    if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors):
+        return False
+    return ops.launch_observer() is None
+
+
+def _weights_bf16(w1, w3, w2, shadows):
+    shadows = shadows or (None, None, None)
+    return [sh if sh is not None else ops.cast_bf16(_dense(w)) for w, sh in zip((w1, w3, w2), shadows)]
+
+
 def moe_ffn(x: torch.Tensor, logits: torch.Tensor, w1: torch.Tensor, w3: torch.Tensor,
             w2: torch.Tensor, k: int, bias: torch.Tensor | None = None, return_routing: bool = False,
             bf16_weights=None, accumulate_into_grad: bool = False):
@@ -304,6 +318,9 @@ def moe_ffn(x: torch.Tensor, logits: torch.Tensor, w1: torch.Tensor, w3: torch.T
     With `return_routing` also returns a dict of the integer routing tensors and gates.
     `bf16_weights`: bf16 copies of (w1, w3, w2) to compute with (None entries are cast here).
     `accumulate_into_grad`: w1, w3, w2 must be leaf tensors; see the module docstring."""
+    if not return_routing and x.shape[0] > 0 and _forward_only(x, logits, w1, w3, w2, bias):
+        w1b, w3b, w2b = _weights_bf16(w1, w3, w2, bf16_weights)
+        return ops.ffn_forward(_dense(x), _dense(logits), w1b, w3b, w2b, k, bias)
     grad_params = None
     if accumulate_into_grad:
         grad_params = tuple(w if (w.requires_grad and w.is_leaf) else None for w in (w1, w3, w2))
@@ -516,6 +533,13 @@ def routed_moe(x: torch.Tensor, router_weight: torch.Tensor, w1: torch.Tensor, w
     whatever the dtypes (the reference's behaviour under its bf16 autocast); the output has
     the dtype of x.  With `return_routing` a dict of the integer routing tensors and gates is
     returned as a third value."""
+    if not return_routing and x.shape[0] > 0 and _forward_only(x, router_weight, w1, w3, w2, bias):
+        # nothing to keep for a backward pass: the router product, then the rest in one call
+        w1b, w3b, w2b = _weights_bf16(w1, w3, w2, bf16_weights)
+        xn = ops.cast_bf16(_dense(x))
+        with torch.autocast("cuda", enabled=False):
+            logits = xn @ router_weight.detach().to(torch.bfloat16).t()
+        return ops.ffn_forward(xn, logits, w1b, w3b, w2b, k, bias, out_dtype=x.dtype), logits
     grad_params = None
     if accumulate_into_grad:
         grad_params = tuple(w if (w.requires_grad and w.is_leaf) else None for w in (w1, w3, w2))

@@ -58,6 +58,9 @@ SIGNATURES = {
                                _i64, _vp]),
     "moe_combine_bwd_by_token": (_int, [_vp, _int, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _vp]),
     "moe_cast_f32_bf16": (_int, [_vp, _vp, _i64, _vp]),
+    "moe_ffn_forward_workspace_bytes": (_i64, [_i64, _i64, _i64, _i64, _i64]),
+    "moe_ffn_forward": (_int, [_vp, _int, _vp, _int, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _int,
+                                _vp, _i64, _vp]),
     "moe_f32_gather_rows": (_int, [_vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp]),
     "moe_f32_combine_fwd": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp]),
     "moe_f32_combine_bwd": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _vp]),

@@ -48,6 +48,11 @@ def _stream():
     return torch.cuda.current_stream().cuda_stream
 
 
+def launch_observer():
+    """The object installed as the library's launch observer (a profiling aid), or None."""
+    return _lib.load().observer
+
+
 def router_topk(logits: torch.Tensor, k: int, bias: torch.Tensor | None = None):
     """logits [T,E] (bf16/fp32) -> ids int32 [T*k], gates fp32 [T*k]."""
     T, E = logits.shape
@@ -375,6 +380,21 @@ def cast_bf16(w: torch.Tensor) -> torch.Tensor:
         return w
     out = torch.empty(w.shape, dtype=torch.bfloat16, device=w.device)
     _lib.load().call("moe_cast_f32_bf16", _p(w), _p(out), w.numel(), _stream())
+    return out
+
+
+def ffn_forward(x: torch.Tensor, logits: torch.Tensor, w1: torch.Tensor, w3: torch.Tensor, w2: torch.Tensor,
+                k: int, bias: torch.Tensor | None = None, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """The layer body's forward pass in one call of the library (no intermediate is kept): x [T,H]
+    bf16/fp32, logits [T,E] bf16/fp32, bf16 weights -> out [T,H] of `out_dtype` (default: x's)."""
+    T, H = x.shape
+    E, I = w1.shape[0], w1.shape[1]
+    L = _lib.load()
+    out = torch.empty(T, H, dtype=out_dtype or x.dtype, device=x.device)
+    nbytes = L.cdll.moe_ffn_forward_workspace_bytes(T, H, E, I, k)
+    ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=x.device)
+    L.call("moe_ffn_forward", _p(x), _dt(x), _p(logits), _dt(logits), _p(bias), _p(w1), _p(w3), _p(w2),
+           T, H, E, I, k, _p(out), _dt(out), _p(ws), ws.numel(), _stream())
     return out
 
 
