@@ -4,7 +4,7 @@
 // dispatch kernels as the bf16 path; what differs is the row type of the expert-contiguous
 // buffers (fp32 [R,H] / [R,I]) and the matrix instruction (v_mfma_f32_32x32x2_f32, fp32
 // operands, fp32 accumulate).  A compatibility mode: correct and bounds-checked, 64 x 64 or
-// 128 x 128 tiles from plain HIP, 60 to 80 % of the fp32 matrix peak on large shapes.
+// 128 x 128 tiles from plain HIP, 75 to 80 % of the fp32 matrix peak on large shapes.
 #include "common.h"
 
 namespace {
@@ -135,22 +135,31 @@ __device__ __forceinline__ void clear(f32x16 (&acc)[Shape<T>::NB][Shape<T>::NB])
 
 // Row-ragged: C[r, :] (+)= A[r, :] x B_e for the rows r of expert e.  A [R,K] row-major;
 // B_e = B + e*N*K holds either [N,K] (B_KCONT: C = A B_e^T, the forward products) or [K,N]
-// (C = A B_e, the input gradients).  blockIdx.x counts T-row tiles over all experts (an
-// expert's last tile may be short), blockIdx.y T-column tiles.
+// (C = A B_e, the input gradients).  Tiles are numbered row tile by row tile (T-row tiles counted
+// over all experts, an expert's last one may be short), column tiles fastest.  The hardware hands
+// workgroup b to XCD b % 8, each with an L2 of its own: XCD x takes the x-th contiguous eighth of
+// the tile list, so that the workgroups it runs side by side share a few row tiles (every column
+// tile of a row tile reads the same rows of A) and one or two experts' weights in its L2.
 template <int T, bool B_KCONT>
 __global__ __launch_bounds__(256) void f32_gemm_rows_kernel(F32Gemm p) {
   constexpr int LD = Shape<T>::LD, PER = Shape<T>::PER, NB = Shape<T>::NB;
   __shared__ __align__(16) float sA[TK * LD], sB[TK * LD];
   __shared__ int s_tile[3];
+  const int n_col = (p.N + T - 1) / T;
+  const long long total = (long long)(p.R / T + p.E) * n_col;  // (the grid's size)
+  const long long chunk = (total + 7) / 8;
+  const long long tile = (long long)(blockIdx.x % 8) * chunk + blockIdx.x / 8;
+  if (blockIdx.x / 8 >= chunk || tile >= total) return;
+  const int row_tile = (int)(tile / n_col), col_tile = (int)(tile % n_col);
   if (threadIdx.x == 0) {
     int seen = 0, found = -1, row0 = 0, row_end = 0;
     for (int e = 0; e < p.E; ++e) {
       const int b = p.offs[e], n = p.offs[e + 1] - b;
       if (n <= 0 || b < 0 || b + n > p.R) continue;  // (empty, or offsets no dispatch would produce)
       const int nt = (n + T - 1) / T;
-      if ((int)blockIdx.x < seen + nt) {
+      if (row_tile < seen + nt) {
         found = e;
-        row0 = b + ((int)blockIdx.x - seen) * T;
+        row0 = b + (row_tile - seen) * T;
         row_end = b + n;
         break;
       }
@@ -162,8 +171,8 @@ __global__ __launch_bounds__(256) void f32_gemm_rows_kernel(F32Gemm p) {
   }
   __syncthreads();
   const int e = s_tile[0], row0 = s_tile[1], row_end = s_tile[2];
-  if (e < 0) return;  // (the grid is sized for the worst case: R/T + E tiles)
-  const int n0 = blockIdx.y * T;
+  if (e < 0) return;  // (the grid is sized for the worst case: R/T + E row tiles)
+  const int n0 = col_tile * T;
   const float* Be = p.B + (long long)e * p.N * p.K;
   const int wv = threadIdx.x >> 6, wm = wv >> 1, wn = wv & 1;
   f32x16 acc[NB][NB];
@@ -188,13 +197,22 @@ __global__ __launch_bounds__(256) void f32_gemm_rows_kernel(F32Gemm p) {
 }
 
 // k-ragged: C_e[m, n] (+)= sum over the rows r of expert e of A[r, m] * B[r, n]  (the weight
-// gradients).  A [R,M], B [R,N] row-major, C [E,M,N].  grid = (N tiles, M tiles, E).  An expert
+// gradients).  A [R,M], B [R,N] row-major, C [E,M,N].  Tiles are numbered expert by expert and an
+// XCD takes a contiguous eighth of them (as in the kernel above): the workgroups an XCD runs side
+// by side then walk the rows of one or two experts together and find them in its L2.  An expert
 // without rows gets zeros (or is left alone when accumulating).
 template <int T>
 __global__ __launch_bounds__(256) void f32_gemm_wgrad_kernel(F32Gemm p) {
   constexpr int LD = Shape<T>::LD, PER = Shape<T>::PER, NB = Shape<T>::NB;
   __shared__ __align__(16) float sA[TK * LD], sB[TK * LD];
-  const int e = blockIdx.z, n0 = blockIdx.x * T, m0 = blockIdx.y * T;
+  const int n_col = (p.N + T - 1) / T, n_row = (p.M + T - 1) / T;
+  const long long total = (long long)p.E * n_row * n_col;
+  const long long chunk = (total + 7) / 8;
+  const long long tile = (long long)(blockIdx.x % 8) * chunk + blockIdx.x / 8;
+  if (blockIdx.x / 8 >= chunk || tile >= total) return;
+  const int e = (int)(tile / ((long long)n_row * n_col));
+  const int in_e = (int)(tile % ((long long)n_row * n_col));
+  const int n0 = (in_e % n_col) * T, m0 = (in_e / n_col) * T;
   int b = p.offs[e], end = p.offs[e + 1];
   if (b < 0 || end > p.R || end < b) b = end = 0;
   const int wv = threadIdx.x >> 6, wm = wv >> 1, wn = wv & 1;
@@ -465,14 +483,15 @@ extern "C" int moe_f32_gemm_rows(const float* a, const float* b, const int32_t* 
   if (!offs) return MOE_ERR_NULL;
   F32Gemm p{a, b, c, offs, (int)E, (int)R, 0, (int)N, (int)K, accumulate};
   hipStream_t s = (hipStream_t)stream;
+  // (one workgroup per tile slot, rounded up to whole eighths: see the kernel's tile numbering)
+  auto blocks = [&](int64_t t) { return (unsigned)(((R / t + E) * ((N + t - 1) / t) + 7) / 8 * 8); };
+  if ((R / 64 + E) * ((N + 63) / 64) + 8 > 0x7fffffffll) return MOE_ERR_LIMIT;
   if (f32_large_tiles((R / 128 + E) * ((N + 127) / 128))) {
-    const dim3 grid((unsigned)(R / 128 + E), (unsigned)((N + 127) / 128));
-    if (b_k_contiguous) hipLaunchKernelGGL((f32_gemm_rows_kernel<128, true>), grid, dim3(256), 0, s, p);
-    else hipLaunchKernelGGL((f32_gemm_rows_kernel<128, false>), grid, dim3(256), 0, s, p);
+    if (b_k_contiguous) hipLaunchKernelGGL((f32_gemm_rows_kernel<128, true>), dim3(blocks(128)), dim3(256), 0, s, p);
+    else hipLaunchKernelGGL((f32_gemm_rows_kernel<128, false>), dim3(blocks(128)), dim3(256), 0, s, p);
   } else {
-    const dim3 grid((unsigned)(R / 64 + E), (unsigned)((N + 63) / 64));
-    if (b_k_contiguous) hipLaunchKernelGGL((f32_gemm_rows_kernel<64, true>), grid, dim3(256), 0, s, p);
-    else hipLaunchKernelGGL((f32_gemm_rows_kernel<64, false>), grid, dim3(256), 0, s, p);
+    if (b_k_contiguous) hipLaunchKernelGGL((f32_gemm_rows_kernel<64, true>), dim3(blocks(64)), dim3(256), 0, s, p);
+    else hipLaunchKernelGGL((f32_gemm_rows_kernel<64, false>), dim3(blocks(64)), dim3(256), 0, s, p);
   }
   return moe_launch_status();
 }
@@ -490,13 +509,12 @@ extern "C" int moe_f32_gemm_wgrad(const float* a, const float* b, const int32_t*
     MOE_CHECK_PTR(b);
   }
   F32Gemm p{a, b, dw, offs, (int)E, (int)R, (int)M, (int)N, 0, accumulate};
-  if (f32_large_tiles(E * ((M + 127) / 128) * ((N + 127) / 128))) {
-    const dim3 grid((unsigned)((N + 127) / 128), (unsigned)((M + 127) / 128), (unsigned)E);
-    hipLaunchKernelGGL(f32_gemm_wgrad_kernel<128>, grid, dim3(256), 0, (hipStream_t)stream, p);
-  } else {
-    const dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64), (unsigned)E);
-    hipLaunchKernelGGL(f32_gemm_wgrad_kernel<64>, grid, dim3(256), 0, (hipStream_t)stream, p);
-  }
+  auto blocks = [&](int64_t t) { return (unsigned)((E * ((M + t - 1) / t) * ((N + t - 1) / t) + 7) / 8 * 8); };
+  if (E * ((M + 63) / 64) * ((N + 63) / 64) + 8 > 0x7fffffffll) return MOE_ERR_LIMIT;
+  if (f32_large_tiles(E * ((M + 127) / 128) * ((N + 127) / 128)))
+    hipLaunchKernelGGL(f32_gemm_wgrad_kernel<128>, dim3(blocks(128)), dim3(256), 0, (hipStream_t)stream, p);
+  else
+    hipLaunchKernelGGL(f32_gemm_wgrad_kernel<64>, dim3(blocks(64)), dim3(256), 0, (hipStream_t)stream, p);
   return moe_launch_status();
 }
 

@@ -79,7 +79,7 @@ class MoE(nn.Module):
         # False (the reference's rule): a call without autocast on fp32 input and fp32 parameters
         # computes in fp32 from end to end, as the reference's bmm's then do (mlp.py:154-157).
         # True: such a call runs on the bf16 matrix cores like every other one (fp32 in and out,
-        # bf16 operands, fp32 accumulation): nine times the throughput, at bf16 precision.
+        # bf16 operands, fp32 accumulation): eight times the throughput, at bf16 precision.
         self.bf16_compute_for_fp32_calls = False
         self._init_expert_weights(config.seed)
 
