@@ -31,25 +31,32 @@ struct F32Gemm {
 };
 
 // T x 16 tile of an operand whose k index is contiguous in memory (element (i, k) at
-// base[i * ld + k]): thread t takes rows t/4 (+64) and the four k values 4*(t%4).., and writes
-// them transposed into the k-major LDS tile.
+// base[i * ld + k]): a thread takes one row (+64) and four consecutive k values, and writes them
+// transposed into the k-major LDS tile.
+// Which row and which k quad of a T x 16 tile thread t takes: lanes 2n and 2n+1 of a half-wave take
+// the two k quads 0,1 (lower half-wave) or 2,3 (upper) of row n, so that the 32 lanes the LDS serves
+// together write their transposed values to 32 different banks (16 rows x 2 quads, rows of
+// 4 * LD bytes with LD = 4 mod 32).
+__device__ __forceinline__ int kcont_row() { return ((threadIdx.x >> 1) & 15) + 16 * (threadIdx.x >> 6); }
+__device__ __forceinline__ int kcont_quad() { return (threadIdx.x & 1) + 2 * ((threadIdx.x >> 5) & 1); }
+
 template <int T>
 __device__ __forceinline__ void load_kcont(f32x4 (&v)[Shape<T>::PER], const float* base, long long ld, int i0,
                                            int i_lim, int k0, int K) {
-  const int k = k0 + (threadIdx.x & 3) * 4;
+  const int k = k0 + kcont_quad() * 4;
 #pragma unroll
   for (int r = 0; r < Shape<T>::PER; ++r) {
-    const int i = i0 + (threadIdx.x >> 2) + 64 * r;
+    const int i = i0 + kcont_row() + 64 * r;
     v[r] = f32x4{0.f, 0.f, 0.f, 0.f};
     if (i < i_lim && k < K) v[r] = *reinterpret_cast<const f32x4*>(base + (long long)i * ld + k);  // (K % 4 == 0)
   }
 }
 template <int T>
 __device__ __forceinline__ void stage_kcont(float* s, const f32x4 (&v)[Shape<T>::PER]) {
-  const int k = (threadIdx.x & 3) * 4;
+  const int k = kcont_quad() * 4;
 #pragma unroll
   for (int r = 0; r < Shape<T>::PER; ++r) {
-    const int i = (threadIdx.x >> 2) + 64 * r;
+    const int i = kcont_row() + 64 * r;
 #pragma unroll
     for (int x = 0; x < 4; ++x) s[(k + x) * Shape<T>::LD + i] = v[r][x];
   }
