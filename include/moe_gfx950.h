@@ -336,7 +336,9 @@ int moe_ffn_forward(const void* x, int x_dtype, const void* logits, int logits_d
  * step of mlp.py:104-169 in fp32 (the three bmm's of :154-157 included) and so do these
  * entry points.  Routing and dispatch are the entries above (fp32 logits).  Expert-contiguous
  * buffers are fp32 here: xp, dyp, dxp, y [R,H]; g, u, act, dact, dg, du [R,I].  H and I must be
- * multiples of 4 (16-byte accesses); weights are the fp32 parameters themselves. */
+ * multiples of 4 (16-byte accesses); weights are the fp32 parameters themselves.  Limits as
+ * above (R <= 2^30, widths <= 65536, E <= 1024 for the GEMMs) and fewer than 2^31 output tiles
+ * of 64 x 64 per GEMM. */
 
 /* mlp.py:104-131 (repeat_interleave + both sorts): xp[pos,:] = x[pos_to_row[pos] / k, :]. */
 int moe_f32_gather_rows(const float* x, const int32_t* pos_to_row, int64_t T, int64_t R, int64_t H,
