@@ -634,3 +634,55 @@ def test_argument_checks_return_codes(pkg, ops):
         ops.router_topk(torch.zeros(2, 4).cuda(), 5)
     with pytest.raises(RuntimeError, match="GPU tensors"):
         ops.router_topk(torch.zeros(2, 4), 2)
+
+
+def test_grouped_gemms_at_the_expert_limit(pkg, ops):
+    """E = 1024, the most experts the grouped GEMMs take (their per-expert tile table lives in LDS):
+    most experts empty, a few with ragged row counts, every bf16 mode and both fp32 GEMMs against
+    per-expert products; E = 1025 is refused before anything is launched."""
+    E, H, I = 1024, 64, 64
+    g_ = torch.Generator().manual_seed(1024)
+    counts = np.zeros(E, dtype=np.int64)
+    for e, n in ((0, 300), (1, 1), (511, 257), (512, 64), (1022, 5), (1023, 129)):
+        counts[e] = n
+    offs_np = np.zeros(E + 1, dtype=np.int32)
+    offs_np[1:] = np.cumsum(counts)
+    R = int(offs_np[-1])
+    offs = torch.from_numpy(offs_np).cuda()
+    bf = torch.bfloat16
+    xp = torch.randn(R, H, generator=g_).to(bf).cuda()
+    dyp = torch.randn(R, H, generator=g_).to(bf).cuda()
+    w1, w3 = ((torch.randn(E, I, H, generator=g_) * 0.2).to(bf).cuda() for _ in range(2))
+    w2 = (torch.randn(E, H, I, generator=g_) * 0.2).to(bf).cuda()
+    gg, uu, act = ops.gemm_gateup(xp, w1, w3, offs, save_gu=True)
+    y = ops.gemm_down(act, w2, offs)
+    dg, du = ops.gemm_dgrad_down(dyp, w2, gg, uu, offs)[:2]
+    dxp = ops.gemm_dgrad_gateup(dg, du, w1, w3, offs)
+    dw2 = ops.gemm_wgrad(dyp, act, offs, E, torch.float32)
+    live = [e for e in range(E) if counts[e]]
+    for e in live:
+        a, b = int(offs_np[e]), int(offs_np[e + 1])
+        xe = xp[a:b].float()
+        ge, ue = xe @ w1[e].float().t(), xe @ w3[e].float().t()
+        assert _close(gg[a:b], ge) and _close(uu[a:b], ue), e
+        assert _close(act[a:b], torch.nn.functional.silu(ge) * ue), e
+        assert _close(y[a:b], act[a:b].float() @ w2[e].float().t()), e
+        assert _close(dxp[a:b], dg[a:b].float() @ w1[e].float() + du[a:b].float() @ w3[e].float()), e
+        ref = dyp[a:b].float().t() @ act[a:b].float()
+        assert ((dw2[e] - ref).norm() / ref.norm().clamp_min(1e-20)).item() < 1e-3, e
+    dead = torch.tensor([e for e in range(E) if not counts[e]]).cuda()
+    assert not dw2[dead].any()
+    # the fp32 entries on the same offsets
+    c32 = ops.f32_gemm_rows(xp.float(), w1.float(), offs, True)
+    w32 = ops.f32_gemm_wgrad(dyp.float(), xp.float(), offs, E)
+    for e in live:
+        a, b = int(offs_np[e]), int(offs_np[e + 1])
+        assert torch.allclose(c32[a:b], xp[a:b].float() @ w1[e].float().t(), rtol=1e-4, atol=1e-4), e
+        assert torch.allclose(w32[e], dyp[a:b].float().t() @ xp[a:b].float(), rtol=1e-4, atol=1e-3), e
+    assert not w32[dead].any()
+    big = torch.zeros(1026, dtype=torch.int32).cuda()
+    wbig = torch.zeros(1025, I, H, dtype=bf).cuda()
+    with pytest.raises(pkg.lib.MoELibError, match="MOE_ERR_LIMIT"):
+        ops.gemm_gateup(xp, wbig, wbig, big, save_gu=False)
+    with pytest.raises(pkg.lib.MoELibError, match="MOE_ERR_LIMIT"):
+        ops.f32_gemm_rows(xp.float(), wbig.float(), big, True)
