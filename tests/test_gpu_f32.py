@@ -316,3 +316,30 @@ def test_f32_layer_is_reproducible_bit_for_bit(P):
     a, b = run(), run()
     for i, (p, q) in enumerate(zip(a, b)):
         assert torch.equal(p, q), i
+
+
+def test_f32_empty_batch_and_masked_experts(P):
+    """The edges of the fp32 path: no tokens at all (exact-zero weight gradients, empty outputs),
+    and logits with -inf (experts masked out for some tokens) selected exactly as the oracle does."""
+    E, H, I, k = 8, 64, 32, 2
+    g = torch.Generator().manual_seed(9)
+    w1, w3 = (torch.randn(E, I, H, generator=g).cuda().requires_grad_(True) for _ in range(2))
+    w2 = torch.randn(E, H, I, generator=g).cuda().requires_grad_(True)
+    x0 = torch.zeros(0, H).cuda().requires_grad_(True)
+    out0 = P.moe_ffn_f32(x0, torch.zeros(0, E).cuda(), w1, w3, w2, k)
+    assert out0.shape == (0, H) and out0.dtype == torch.float32
+    out0.sum().backward()
+    assert x0.grad.shape == (0, H)
+    for w in (w1, w3, w2):
+        assert w.grad is not None and not w.grad.any()
+    T = 50
+    x = torch.randn(T, H, generator=g)
+    logits = torch.randn(T, E, generator=g)
+    logits[::3, :5] = float("-inf")          # three finite logits left
+    logits[1::7, :7] = float("-inf")         # one finite logit for k = 2: the second slot's gate is 0
+    out, rt = P.moe_ffn_f32(x.cuda(), logits.cuda(), w1.detach(), w3.detach(), w2.detach(), k, return_routing=True)
+    f = O.moe_forward(x, torch.zeros(E, H), w1.detach().cpu(), w3.detach().cpu(), w2.detach().cpu(), k,
+                      logits=logits.double(), compute_dtype=torch.float64)
+    assert np.array_equal(rt["ids"].cpu().numpy().reshape(T, k), f["ids"].astype(np.int32))
+    assert torch.isfinite(out).all()
+    _close("out with masked experts", out, f["out"])
