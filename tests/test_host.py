@@ -261,3 +261,21 @@ def test_sizes_and_dtypes_are_checked_before_any_launch():
                 assert call(i, 7) == -4, f"{name}: dtype code 7 for {n} not refused as MOE_ERR_DTYPE"
                 checked += 1
     assert checked > 100
+
+
+def test_precision_rule_of_the_module_cpu():
+    """Which calls the module runs in fp32 from end to end: those the reference would (fp32 input,
+    fp32 parameters, no autocast), unless the caller asks for the bf16 cores."""
+    pkg = load_pkg()
+    cfg = pkg.ModelConfig(hidden_size=64, num_experts=4, num_experts_per_tok=2, moe_intermediate_size=32)
+    m = pkg.MoE(cfg)
+    x = torch.zeros(1, 2, 64)
+    assert m._runs_in_fp32(x)
+    assert not m._runs_in_fp32(x.to(torch.bfloat16))
+    m.bf16_compute_for_fp32_calls = True
+    assert not m._runs_in_fp32(x)
+    m.bf16_compute_for_fp32_calls = False
+    mb = pkg.MoE(cfg).to(torch.bfloat16)
+    assert not mb._runs_in_fp32(x) and not mb._runs_in_fp32(x.to(torch.bfloat16))
+    m.experts_up_weights.data = m.experts_up_weights.data.to(torch.bfloat16)   # mixed parameters
+    assert not m._runs_in_fp32(x)
