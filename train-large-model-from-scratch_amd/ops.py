@@ -400,6 +400,11 @@ def ffn_forward(x: torch.Tensor, logits: torch.Tensor, w1: torch.Tensor, w3: tor
 
 # ---- the path in fp32 (layer called without autocast on fp32 tensors) ---------------------------
 
+def _check_offs(offs: torch.Tensor, E: int):
+    if offs.dtype != torch.int32 or offs.numel() != E + 1:
+        raise ValueError(f"offs must be int32 [E + 1] = [{E + 1}], got {offs.dtype} {tuple(offs.shape)}")
+
+
 def _f32(*ts):
     for t in ts:
         if t is not None and t.dtype != torch.float32:
@@ -469,6 +474,9 @@ def f32_gemm_rows(a: torch.Tensor, b: torch.Tensor, offs: torch.Tensor, transpos
     N = b.shape[1] if transpose_b else b.shape[2]
     if (b.shape[2] if transpose_b else b.shape[1]) != K:
         raise ValueError(f"depth mismatch: a {tuple(a.shape)}, b {tuple(b.shape)}, transpose_b={transpose_b}")
+    _check_offs(offs, E)
+    if out is not None and tuple(out.shape) != (R, N):
+        raise ValueError(f"out has shape {tuple(out.shape)}, the product {(R, N)}")
     c = out if out is not None else torch.empty(R, N, dtype=torch.float32, device=a.device)
     _lib.load().call("moe_f32_gemm_rows", _p(a), _p(b), _p(offs), E, R, N, K, int(transpose_b), _p(c),
                      int(out is not None), _stream())
@@ -481,6 +489,10 @@ def f32_gemm_wgrad(a: torch.Tensor, b: torch.Tensor, offs: torch.Tensor, E: int,
     _f32(a, b, out)
     R, M = a.shape
     N = b.shape[1]
+    _check_offs(offs, E)
+    if b.shape[0] != R or (out is not None and tuple(out.shape) != (E, M, N)):
+        raise ValueError(f"shape mismatch: a {tuple(a.shape)}, b {tuple(b.shape)}, E {E}"
+                         + ("" if out is None else f", out {tuple(out.shape)}"))
     dw = out if out is not None else torch.empty(E, M, N, dtype=torch.float32, device=a.device)
     _lib.load().call("moe_f32_gemm_wgrad", _p(a), _p(b), _p(offs), E, R, M, N, _p(dw), int(out is not None),
                      _stream())
