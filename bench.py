@@ -28,13 +28,13 @@ HBM_PEAK_GBS = 8000.0
 # are in profiles/grouped_gemm_cfg3_pmc.txt.  bench.py cannot run the profiler on itself, so
 # the figures are carried here and refreshed whenever that profile is.
 MEASURED_HBM_BYTES_PER_LAUNCH = {
-    (3, "gemm_gateup_swiglu_fwd_blocked"): 3.994e9,
-    (3, "gemm_gateup_swiglu_fwd"): 3.994e9,
-    (3, "gemm_down_fwd"): 1.860e9,
-    (3, "gemm_dgrad_down_swiglu_bwd_blocked"): 2.460e9,
-    (3, "gemm_dgrad_down_swiglu_bwd"): 2.460e9,
-    (3, "gemm_dgrad_gateup_packed"): 3.763e9,
-    (3, "gemm_dgrad_gateup"): 3.763e9,
+    (3, "gemm_gateup_swiglu_fwd_blocked"): 3.980e9,
+    (3, "gemm_gateup_swiglu_fwd"): 3.980e9,
+    (3, "gemm_down_fwd"): 1.813e9,
+    (3, "gemm_dgrad_down_swiglu_bwd_blocked"): 2.450e9,
+    (3, "gemm_dgrad_down_swiglu_bwd"): 2.450e9,
+    (3, "gemm_dgrad_gateup_packed"): 3.790e9,
+    (3, "gemm_dgrad_gateup"): 3.790e9,
     (3, "gemm_wgrad_down"): 1.074e9,
     (3, "gemm_wgrad"): 1.074e9,
     (3, "gemm_wgrad_pair"): 2.18e9,                # from the average over both weight-gradient launches
