@@ -706,7 +706,10 @@ def main():
     if args.config == 3 and not args.no_others:
         others = []
         for cid, fraction in ((1, 1.0), (2, 1.0), (4, 1.0)):
-            rec = time_layer_config(P, torch, dev, cid, max(args.steps // 2, 5), args.warmup)
+            # (the two small configurations take well under a millisecond per step: more steps, so
+            # that one hiccup of the host does not show in their wall-clock mean)
+            n_steps = max(args.steps * 2, 40) if cid in (1, 2) else max(args.steps // 2, 5)
+            rec = time_layer_config(P, torch, dev, cid, n_steps, args.warmup)
             if not args.no_cpu:
                 rec["cpu_baseline"] = cpu_leg(P, torch, cid, fraction)
             others.append(rec)
