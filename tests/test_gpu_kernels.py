@@ -686,3 +686,39 @@ def test_grouped_gemms_at_the_expert_limit(pkg, ops):
         ops.gemm_gateup(xp, wbig, wbig, big, save_gu=False)
     with pytest.raises(pkg.lib.MoELibError, match="MOE_ERR_LIMIT"):
         ops.f32_gemm_rows(xp.float(), wbig.float(), big, True)
+
+
+@pytest.mark.parametrize("counts,M,N", [
+    ([2700, 300], 4096, 2560),                    # 10 groups of 32 tiles for 8 XCDs, one expert with 90 % of the rows
+    ([5, 0, 1900, 40, 0, 700, 64, 3], 2048, 1024),  # one group per expert, two experts empty
+    ([300] * 7 + [2100], 1024, 2048),             # one heavy expert at the end of the list
+])
+def test_weight_gradient_under_skewed_routing(ops, counts, M, N):
+    """The weight-gradient kernel deals its tiles to the XCDs longest first when the routing is
+    skewed (at most 64 experts, whole groups of tiles per expert): every tile must still be
+    computed exactly once, whichever workgroup gets it.  Checked against per-expert products,
+    for both output dtypes and with accumulation."""
+    _say("wgrad skew", counts, M, N)
+    E, R = len(counts), int(sum(counts))
+    offs_np = np.zeros(E + 1, dtype=np.int32)
+    offs_np[1:] = np.cumsum(counts)
+    offs = torch.from_numpy(offs_np).cuda()
+    g_ = torch.Generator().manual_seed(M + N + E)
+    a = torch.randn(R, M, generator=g_).to(torch.bfloat16).cuda()
+    b = torch.randn(R, N, generator=g_).to(torch.bfloat16).cuda()
+    dw = ops.gemm_wgrad(a, b, offs, E, torch.float32)
+    dwb = ops.gemm_wgrad(a, b, offs, E, torch.bfloat16)
+    prev = torch.randn(E, M, N, generator=g_).cuda()
+    acc = prev.clone()
+    ops.gemm_wgrad(a, b, offs, E, torch.float32, out=acc)
+    for e in range(E):
+        s, t = int(offs_np[e]), int(offs_np[e + 1])
+        ref = a[s:t].float().t() @ b[s:t].float()
+        if s == t:
+            assert not dw[e].any() and not dwb[e].any() and torch.equal(acc[e], prev[e])
+            continue
+        assert ((dw[e] - ref).norm() / ref.norm()).item() < 1e-3, e
+        assert ((dwb[e].float() - ref).norm() / ref.norm()).item() < 5e-3, e
+        assert (((acc[e] - prev[e]) - ref).norm() / ref.norm()).item() < 1e-3, e
+    dw2 = ops.gemm_wgrad(a, b, offs, E, torch.float32)
+    assert torch.equal(dw, dw2)
