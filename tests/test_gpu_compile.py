@@ -38,8 +38,8 @@ def test_registered_operators_pass_opcheck(pkg, lib):
     torch.library.opcheck(traced.ffn_fwd, args,
                           test_utils=("test_schema", "test_faketensor", "test_autograd_registration"))
     outs = traced.ffn_fwd(*[a.detach() if isinstance(a, torch.Tensor) else a for a in args])
-    out, ids, gates, offs, p2r, r2p, xp, g, u, act, w1b, w3b, w2b = outs
-    bargs = (torch.randn_like(out), xp, g, u, act, gates, ids, offs, p2r, r2p, w1b, w3b, w2b, 2, True, False, True)
+    out, ids, gates, offs, p2r, r2p, xp, gu, act, w1b, w3b, w2b = outs
+    bargs = (torch.randn_like(out), xp, gu, act, gates, ids, offs, p2r, r2p, w1b, w3b, w2b, 2, True, False, True)
     torch.library.opcheck(traced.ffn_bwd, bargs, test_utils=("test_schema", "test_faketensor"))
 
 

@@ -92,17 +92,30 @@ def test_registered_operators_propagate_shapes_without_a_gpu():
             for train in (True, False):
                 o = traced.ffn_fwd(x, lg, *ws, k, train)
                 shapes = [tuple(t.shape) for t in o]
-                gu = (T * k, I) if train else (0,)
+                gu = (traced.gu_blocked_bytes(T * k, E, I),) if train else (0,)
                 cp = [tuple(w.shape) if wdt == f32 else (0,) for w in ws]
-                assert shapes == [(T, H), (T * k,), (T * k,), (E + 1,), (T * k,), (T * k,), (T * k, H), gu, gu,
+                assert shapes == [(T, H), (T * k,), (T * k,), (E + 1,), (T * k,), (T * k,), (T * k, H), gu,
                                   (T * k, I)] + cp
                 assert [t.dtype for t in o[:6]] == [f32, i32, f32, i32, i32, i32]
-                assert all(t.dtype == bf for t in o[6:])
-            out, ids, gates, offs, p2r, r2p, xp, g, u, act, w1b, w3b, w2b = traced.ffn_fwd(x, lg, *ws, k, True)
+                assert o[7].dtype == torch.uint8 and all(t.dtype == bf for t in o[6:7] + o[8:])
+            out, ids, gates, offs, p2r, r2p, xp, gu, act, w1b, w3b, w2b = traced.ffn_fwd(x, lg, *ws, k, True)
             wb = ws if wdt == bf else [w1b, w3b, w2b]
-            d = traced.ffn_bwd(out, xp, g, u, act, gates, ids, offs, p2r, r2p, *wb, k, True, False, wdt == f32)
+            d = traced.ffn_bwd(out, xp, gu, act, gates, ids, offs, p2r, r2p, *wb, k, True, False, wdt == f32)
             assert [tuple(t.shape) for t in d] == [(T, H), (T, E)] + [tuple(w.shape) for w in ws]
             assert [t.dtype for t in d] == [f32, bf, wdt, wdt, wdt]
+
+
+def test_traced_buffer_size_is_the_library_s(lib):
+    """The size the traced forward operator's shape function gives the blocked g/u buffer is the
+    one the library reports (and the wrapper allocates), over ragged and empty shapes."""
+    import importlib
+
+    from conftest import PKG_NAME
+    traced = importlib.import_module(PKG_NAME + ".traced")
+    for R in (0, 1, 255, 256, 257, 4096, 131072, 131073):
+        for E in (1, 8, 64, 1024):
+            for I in (32, 48, 1024, 1056):
+                assert traced.gu_blocked_bytes(R, E, I) == max(lib.cdll.moe_gu_blocked_bytes(R, E, I), 16)
 
 
 def test_mfu_table_for_amd_parts(monkeypatch):

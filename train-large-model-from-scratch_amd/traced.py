@@ -24,7 +24,7 @@ import torch
 from torch import Tensor
 
 from . import ops
-from .functional import _gemm_wgrad
+from .functional import _expert_backward
 
 _BF16 = torch.bfloat16
 
@@ -33,12 +33,21 @@ def _empty(ref: Tensor, dtype=_BF16) -> Tensor:
     return torch.empty(0, dtype=dtype, device=ref.device)
 
 
+def gu_blocked_bytes(R, E: int, I: int):
+    """Size of ops.gemm_gateup_blocked's buffer, as arithmetic a symbolic row count passes through:
+    moe_gu_blocked_bytes (4 KB per 32 x 32 block of ceil(R/256) + E row tiles of 256 rows), with
+    the wrapper's floor of 16 bytes."""
+    return (((R + 255) // 256 + E) * 8 * ((I + 31) // 32) * 4096) if R > 0 else 16
+
+
 @torch.library.custom_op("moe_gfx950::ffn_fwd", mutates_args=(), device_types="cuda")
 def ffn_fwd(x: Tensor, logits: Tensor, w1: Tensor, w3: Tensor, w2: Tensor, k: int,
             train: bool) -> tuple[Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor,
-                                  Tensor, Tensor, Tensor, Tensor, Tensor]:
-    """-> out, ids, gates, offs, pos_to_row, row_to_pos, xp, g, u, act, w1b, w3b, w2b.
-    Without `train` g and u are empty; a weight that already is bf16 has an empty copy."""
+                                  Tensor, Tensor, Tensor, Tensor]:
+    """-> out, ids, gates, offs, pos_to_row, row_to_pos, xp, gu, act, w1b, w3b, w2b.
+    `gu` holds g and u in the library's blocked layout (an opaque uint8 buffer that only the
+    backward operator reads; empty without `train`); a weight that already is bf16 has an empty
+    copy."""
     T, H = x.shape
     E = logits.shape[1]
     x, logits = ops.dense(x), ops.dense(logits)
@@ -46,13 +55,14 @@ def ffn_fwd(x: Tensor, logits: Tensor, w1: Tensor, w3: Tensor, w2: Tensor, k: in
     ids, gates = ops.router_topk(logits, k, None)
     _, offs, pos_to_row, row_to_pos = ops.histogram_scan(ids, E)
     xp = ops.permute_fwd(x, pos_to_row, k, row_to_pos)
-    g, u, act = ops.gemm_gateup(xp, wb[0], wb[1], offs, save_gu=train)
+    if train:
+        gu, act = ops.gemm_gateup_blocked(xp, wb[0], wb[1], offs)
+    else:
+        gu, act = _empty(x, torch.uint8), ops.gemm_gateup(xp, wb[0], wb[1], offs, save_gu=False)[2]
     y = ops.gemm_down(act, wb[2], offs)
     out = ops.combine_fwd(y, gates, row_to_pos, T, k, x.dtype)
-    if not train:
-        g, u = _empty(x), _empty(x)
     copies = [b if w.dtype != _BF16 else _empty(x) for w, b in zip((w1, w3, w2), wb)]
-    return (out, ids, gates, offs, pos_to_row, row_to_pos, xp, g, u, act, *copies)
+    return (out, ids, gates, offs, pos_to_row, row_to_pos, xp, gu, act, *copies)
 
 
 @ffn_fwd.register_fake
@@ -62,18 +72,19 @@ def _(x, logits, w1, w3, w2, k, train):
     R = T * k
     i32 = lambda *s: x.new_empty(s, dtype=torch.int32)
     b16 = lambda *s: x.new_empty(s, dtype=_BF16)
-    gu = (R, I) if train else (0,)
+    gu_bytes = gu_blocked_bytes(R, E, I) if train else 0
     copies = [b16(*w.shape) if w.dtype != _BF16 else b16(0) for w in (w1, w3, w2)]
     return (x.new_empty(T, H), i32(R), x.new_empty(R, dtype=torch.float32), i32(E + 1), i32(R), i32(R),
-            b16(R, H), b16(*gu), b16(*gu), b16(R, I), *copies)
+            b16(R, H), x.new_empty(gu_bytes, dtype=torch.uint8), b16(R, I), *copies)
 
 
 @torch.library.custom_op("moe_gfx950::ffn_bwd", mutates_args=(), device_types="cuda")
-def ffn_bwd(dout: Tensor, xp: Tensor, g: Tensor, u: Tensor, act: Tensor, gates: Tensor,
+def ffn_bwd(dout: Tensor, xp: Tensor, gu: Tensor, act: Tensor, gates: Tensor,
             ids: Tensor, offs: Tensor, pos_to_row: Tensor, row_to_pos: Tensor, w1b: Tensor,
             w3b: Tensor, w2b: Tensor, k: int, x_is_f32: bool, logits_is_f32: bool,
             w_is_f32: bool) -> tuple[Tensor, Tensor, Tensor, Tensor, Tensor]:
-    """-> dx, dlogits, dw1, dw3, dw2."""
+    """-> dx, dlogits, dw1, dw3, dw2.  The kernels of the eager backward pass
+    (`functional._expert_backward`)."""
     T = dout.shape[0]
     E = offs.numel() - 1
     f32 = torch.float32
@@ -81,21 +92,16 @@ def ffn_bwd(dout: Tensor, xp: Tensor, g: Tensor, u: Tensor, act: Tensor, gates: 
     if dout.dtype not in (_BF16, f32):
         dout = dout.float()
     dyp, _ = ops.combine_bwd(dout, None, gates, pos_to_row, k, row_to_pos)
-    dg, du, part = ops.gemm_dgrad_down(dyp, w2b, g, u, offs, dgate_blocks=True)
-    dgates = ops.dgates_from_blocks(part, gates, row_to_pos, pos_to_row)
-    dxp = ops.gemm_dgrad_gateup(dg, du, w1b, w3b, offs)
     wdt = f32 if w_is_f32 else _BF16
-    segs = {}
-    dw2 = _gemm_wgrad(dyp, act, offs, E, wdt, segs=segs)
-    dw1 = _gemm_wgrad(dg, xp, offs, E, wdt, segs=segs)
-    dw3 = _gemm_wgrad(du, xp, offs, E, wdt, segs=segs)
+    dxp, dw1, dw3, dw2, part = _expert_backward(dyp, xp, gu, act, w1b, w3b, w2b, offs, wdt, gate_blocks=True)
+    dgates = ops.dgates_from_blocks(part, gates, row_to_pos, pos_to_row)
     dx = ops.permute_bwd(dxp, row_to_pos, T, k, f32 if x_is_f32 else _BF16)
     dlogits = ops.router_topk_bwd(gates, dgates, ids, T, E, k, f32 if logits_is_f32 else _BF16)
     return dx, dlogits, dw1, dw3, dw2
 
 
 @ffn_bwd.register_fake
-def _(dout, xp, g, u, act, gates, ids, offs, pos_to_row, row_to_pos, w1b, w3b, w2b, k, x_is_f32,
+def _(dout, xp, gu, act, gates, ids, offs, pos_to_row, row_to_pos, w1b, w3b, w2b, k, x_is_f32,
       logits_is_f32, w_is_f32):
     T, H = dout.shape
     E = offs.shape[0] - 1
@@ -109,10 +115,10 @@ def _(dout, xp, g, u, act, gates, ids, offs, pos_to_row, row_to_pos, w1b, w3b, w
 
 def _setup_context(ctx, inputs, output):
     x, logits, w1, w3, w2, k, train = inputs
-    out, ids, gates, offs, pos_to_row, row_to_pos, xp, g, u, act, w1b, w3b, w2b = output
+    out, ids, gates, offs, pos_to_row, row_to_pos, xp, gu, act, w1b, w3b, w2b = output
     # the bf16 operands: the copy made in the forward, or the weight itself
     wb = [w if w.dtype == _BF16 else b for w, b in zip((w1, w3, w2), (w1b, w3b, w2b))]
-    ctx.save_for_backward(xp, g, u, act, gates, ids, offs, pos_to_row, row_to_pos, *wb)
+    ctx.save_for_backward(xp, gu, act, gates, ids, offs, pos_to_row, row_to_pos, *wb)
     ctx.k, ctx.train = k, train
     ctx.flags = (x.dtype == torch.float32, logits.dtype == torch.float32, w1.dtype == torch.float32)
 
@@ -120,8 +126,8 @@ def _setup_context(ctx, inputs, output):
 def _backward(ctx, dout, *unused):
     if not ctx.train:
         raise RuntimeError("moe_gfx950::ffn_fwd was called with train=False: nothing was saved for backward")
-    xp, g, u, act, gates, ids, offs, pos_to_row, row_to_pos, w1b, w3b, w2b = ctx.saved_tensors
-    dx, dlogits, dw1, dw3, dw2 = ffn_bwd(dout, xp, g, u, act, gates, ids, offs, pos_to_row, row_to_pos,
+    xp, gu, act, gates, ids, offs, pos_to_row, row_to_pos, w1b, w3b, w2b = ctx.saved_tensors
+    dx, dlogits, dw1, dw3, dw2 = ffn_bwd(dout, xp, gu, act, gates, ids, offs, pos_to_row, row_to_pos,
                                          w1b, w3b, w2b, ctx.k, *ctx.flags)
     return dx, dlogits, dw1, dw3, dw2, None, None
 
