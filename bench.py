@@ -399,6 +399,34 @@ def module_config3(P, torch, dev, steps, warmup):
         ms = (time.perf_counter() - t0) * 1e3 / steps
         out[name] = {"ms_per_step": round(ms, 4), "tflops": round(flops / ms / 1e9, 1),
                      "tokens_per_s": round(s.T / (ms * 1e-3), 1)}
+    # the same fresh step with the module under `torch.compile` (the reference's --use_compile,
+    # trainer.py:130-131, default backend): the layer body is the pair of registered operators,
+    # which cast the fp32 expert weights in every forward as the reference does
+    try:
+        m.accumulate_wgrad_into_grad = False
+        cm = torch.compile(m, fullgraph=True)
+
+        def cstep():
+            m.zero_grad(set_to_none=True)
+            x.grad = None
+            with torch.autocast("cuda", dtype=torch.bfloat16):
+                o, _ = cm(x)
+            o.backward(dy)
+
+        for _ in range(max(warmup, 2)):
+            cstep()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            cstep()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / steps
+        out["fresh_grads_torch_compile"] = {"ms_per_step": round(ms, 4), "tflops": round(flops / ms / 1e9, 1),
+                                            "tokens_per_s": round(s.T / (ms * 1e-3), 1)}
+        del cm
+    except Exception as e:  # a broken compiler stack on the box must not cost the benchmark line
+        out["fresh_grads_torch_compile"] = {"error": repr(e)[:300]}
+    torch._dynamo.reset()
     del m
     torch.cuda.empty_cache()
     return {"config": 3, "workload": s.name + ", MoE module with fp32 master weights and fp32 input under bf16 "
