@@ -103,6 +103,29 @@ def test_registered_operators_propagate_shapes_without_a_gpu():
             d = traced.ffn_bwd(out, xp, gu, act, gates, ids, offs, p2r, r2p, *wb, k, True, False, wdt == f32)
             assert [tuple(t.shape) for t in d] == [(T, H), (T, E)] + [tuple(w.shape) for w in ws]
             assert [t.dtype for t in d] == [f32, bf, wdt, wdt, wdt]
+            # the pair with the router product inside: bf16 copies only of what is not bf16 already
+            for xdt in (f32, bf):
+                xr = torch.empty(T, H, device="cuda", dtype=xdt)
+                wr = torch.empty(E, H, device="cuda", dtype=wdt)
+                for train in (True, False):
+                    o = traced.routed_fwd(xr, wr, *ws, k, train)
+                    R = T * k
+                    kept = lambda shape, made: tuple(shape) if (train and made) else (0,)
+                    assert [tuple(t.shape) for t in o] == [
+                        (T, H), (T, E), (R,), (R,), (E + 1,), (R,), (R,), kept((T, H), xdt == f32),
+                        kept((E, H), wdt == f32), kept((R, H), True),
+                        (traced.gu_blocked_bytes(R, E, I) if train else 0,), kept((R, I), True)] + [
+                        tuple(w.shape) if wdt == f32 else (0,) for w in ws]
+                    assert [t.dtype for t in o[:7]] == [xdt, bf, i32, f32, i32, i32, i32]
+                    assert o[10].dtype == torch.uint8 and all(t.dtype == bf for t in o[7:10] + o[11:])
+                (out, logits, ids, gates, offs, p2r, r2p, xn, wrb, xp, gu, act, w1b, w3b, w2b) = traced.routed_fwd(
+                    xr, wr, *ws, k, True)
+                wb = ws if wdt == bf else [w1b, w3b, w2b]
+                for ext in (None, logits):
+                    d = traced.routed_bwd(out, ext, xr if xdt == bf else xn, wr if wdt == bf else wrb, xp, gu, act,
+                                          gates, ids, offs, p2r, r2p, *wb, k, xdt == f32, wdt == f32, wdt == f32)
+                    assert [tuple(t.shape) for t in d] == [(T, H), (E, H)] + [tuple(w.shape) for w in ws]
+                    assert [t.dtype for t in d] == [xdt, wdt, wdt, wdt, wdt]
 
 
 def test_traced_buffer_size_is_the_library_s(lib):

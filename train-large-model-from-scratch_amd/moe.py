@@ -197,6 +197,11 @@ class MoE(nn.Module):
         if torch.compiler.is_compiling():
             # under torch.compile (trainer.py:130-131): the same kernels as registered
             # operators the tracer can keep in the graph (traced.py); no cached weight copies
+            if self._router_in_bf16(x):
+                out, gate_logits = traced.routed_moe(x.reshape(B * T, D), self.router.weight,
+                                                     self.experts_gate_weights, self.experts_up_weights,
+                                                     self.experts_down_weights, self.top_k)
+                return out.reshape(B, T, D), gate_logits.reshape(B, T, self.num_experts)
             gate_logits = nn.functional.linear(x, self.router.weight)
             out = traced.moe_ffn(x.reshape(B * T, D), gate_logits.reshape(B * T, self.num_experts),
                                  self.experts_gate_weights, self.experts_up_weights,
