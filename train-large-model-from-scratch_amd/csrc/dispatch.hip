@@ -823,7 +823,7 @@ extern "C" int moe_combine_bwd_by_token(const void* dy, int dy_dtype, const uint
   if (!row_to_pos) return MOE_ERR_NULL;
   if ((dgates != nullptr) != (y != nullptr)) return MOE_ERR_NULL;
   if (T < 0 || H <= 0 || k <= 0 || (H % 8) != 0) return MOE_ERR_SHAPE;
-  if (T * k > (int64_t)1 << 30 || H > 2048) return MOE_ERR_LIMIT;
+  if (T * k > (int64_t)1 << 30 || H > 2048 || k > MOE_MAX_TOPK) return MOE_ERR_LIMIT;
   hipStream_t s = (hipStream_t)stream;
   if (dy_dtype == MOE_DT_BF16)
     return launch_combine_bwd_token<uint16_t>(dy, y, gates, row_to_pos, T, H, k, dyp, dgates, s);
