@@ -81,3 +81,67 @@ def test_captured_forward_backward_replays_match_eager(pkg, lib, split_wgrad):
         for p, g in zip(params, got[3:]):
             p.grad = g
     del graph
+
+
+def test_captured_step_follows_the_master_weights(pkg, lib):
+    """fp32 master weights change between replays (an optimizer step outside the graph): the graph
+    must round them again on every replay instead of replaying with the bf16 copies the module
+    held when it was captured."""
+    E, H, I, k = 8, 256, 128, 2
+    cfg = pkg.ModelConfig(hidden_size=H, num_experts=E, num_experts_per_tok=k, moe_intermediate_size=I,
+                          init_std=0.05)
+    m = pkg.MoE(cfg, k)
+    gen = torch.Generator().manual_seed(67)
+    x = torch.randn(2, 96, H, generator=gen).cuda()
+    dy = torch.randn(2, 96, H, generator=gen).cuda()
+    params = list(m.parameters())
+
+    def eager():
+        for p in params:
+            p.grad = None
+        xi = x.clone().requires_grad_(True)
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            out, logits = m(xi)
+        out.backward(dy)
+        return [out.detach().clone(), logits.detach().clone(), xi.grad.clone()] + [p.grad.clone() for p in params]
+
+    sx = x.clone().requires_grad_(True)
+
+    def step():
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            out, logits = m(sx)
+        out.backward(dy)
+        return out, logits
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):  # (leaves fresh bf16 copies in the module's cache)
+            for p in params:
+                p.grad = None
+            sx.grad = None
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    for p in params:
+        p.grad = None
+    sx.grad = None
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        s_out, s_logits = step()
+    names = ["out", "gate_logits", "dx"] + [n for n, _ in m.named_parameters()]
+    for rep in range(3):
+        if rep:
+            with torch.no_grad():  # what an optimizer step does: in-place updates of the masters
+                for p in params:
+                    p.add_(0.02 * torch.randn(p.shape, generator=gen).cuda())
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [s_out.clone(), s_logits.clone(), sx.grad.clone()] + [p.grad.clone() for p in params]
+        held = [p.grad for p in params]
+        ref = eager()
+        for n, a, b in zip(names, got, ref):
+            assert torch.equal(a, b), (rep, n)
+        _say(f"  replay {rep} after {'an update of' if rep else 'capturing with'} the masters: identical to eager")
+        for p, g in zip(params, held):
+            p.grad = g
+    del graph

@@ -80,9 +80,11 @@ def _router_wgrad(dlogits, x, w_dtype):
     if offs is None:  # constant for a given token count: made once
         step = (T + S - 1) // S
         offs = torch.clamp(torch.arange(S + 1, device=x.device, dtype=torch.int32) * step, max=T).to(torch.int32)
-        if len(_split_offsets) > 64:
-            _split_offsets.clear()
-        _split_offsets[key] = offs
+        # (not kept when made under graph capture: such a tensor lives in the graph's memory and is
+        # only filled when the graph runs)
+        # (entries are never dropped: a captured graph may be reading one; each is at most 129 ints)
+        if not torch.cuda.is_current_stream_capturing() and len(_split_offsets) < 4096:
+            _split_offsets[key] = offs
     part = ops.gemm_wgrad(_dense(dlogits), _dense(x), offs, S, torch.float32)
     return part.sum(0).to(w_dtype)
 

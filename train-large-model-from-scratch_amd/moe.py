@@ -122,14 +122,19 @@ class MoE(nn.Module):
         `p.data.copy_`, an optimizer that is not a `torch.optim.Optimizer`) are the one case this
         cannot see: `invalidate_weight_cache()` is there for them, `cache_bf16_weights = False`
         turns the cache off, and `verify_weight_cache = True` detects a stale copy.  The copies are handed to the
-        expert function together with the masters: the masters receive the gradients."""
+        expert function together with the masters: the masters receive the gradients.
+        While the stream is being captured into a graph the cache is neither read nor written: the
+        casts are recorded with the rest of the step, so every replay rounds the masters as they
+        are then (a copy that was fresh at capture time would be stale after the first optimizer
+        step, and no Python runs at a replay to notice)."""
         out = []
+        capturing = torch.cuda.is_available() and torch.cuda.is_current_stream_capturing()
         for name in ("experts_gate_weights", "experts_up_weights", "experts_down_weights"):
             w = getattr(self, name)
             if w.dtype == torch.bfloat16:
                 out.append(None)
                 continue
-            if not self.cache_bf16_weights:
+            if not self.cache_bf16_weights or capturing:
                 out.append(None)  # the expert function casts
                 continue
             key = (w._version, _optimizer_steps[0], w.data_ptr(), w.device)
