@@ -957,3 +957,23 @@ def test_forward_only_call_gives_the_bits_of_the_differentiable_one(P, x_dtype, 
     out_m = P.moe_ffn(x, lg_f, w1, w3, w2, k, bias=b)
     out_mg = P.moe_ffn(xg, lg_f, w1, w3, w2, k, bias=b)
     assert torch.equal(out_m, out_mg.detach()) and torch.equal(out_m, out_f)
+
+
+@pytest.mark.parametrize("entry", ENTRIES)
+def test_second_order_gradients_are_refused(P, entry):
+    """The backward pass runs kernels autograd cannot see through: asking for a gradient of a
+    gradient must raise instead of returning a tensor that silently lacks those terms."""
+    g = torch.Generator().manual_seed(3)
+    T, H, I, E, k = 32, 64, 64, 4, 2
+    x = torch.randn(T, H, generator=g).bfloat16().cuda().requires_grad_(True)
+    wr = (torch.randn(E, H, generator=g) * 0.1).bfloat16().cuda().requires_grad_(True)
+    ws = [(torch.randn(s, generator=g) * 0.1).bfloat16().cuda().requires_grad_(True)
+          for s in ((E, I, H), (E, I, H), (E, H, I))]
+    if entry == "moe_ffn":
+        out = P.moe_ffn(x, F.linear(x, wr), *ws, k)
+    else:
+        out = P.routed_moe(x, wr, *ws, k)[0]
+    with pytest.raises(RuntimeError, match="not differentiable"):
+        torch.autograd.grad(out.float().sum(), x, create_graph=True)
+    (dx,) = torch.autograd.grad(out.float().sum(), x)  # the first-order gradient is there as ever
+    assert dx.shape == x.shape and not dx.requires_grad

@@ -41,6 +41,15 @@ from . import ops
 from .ops import dense as _dense
 
 
+def _first_order_only():
+    """Called at the top of every backward here.  The backward passes run kernels autograd cannot
+    see through, so a gradient of a gradient would silently lack their terms: refuse to build a
+    graph over them (grad mode is on inside a backward pass only under `create_graph=True`)."""
+    if torch.is_grad_enabled():
+        raise RuntimeError("the MoE kernels' backward pass is not differentiable: call backward()/grad() "
+                           "without create_graph=True")
+
+
 _SPLIT_ROWS = 512  # tokens per partial sum of the router weight gradient
 _split_offsets = {}  # (tokens, slices, device) -> int32 slice bounds
 
@@ -55,6 +64,7 @@ class _RouterLinear(torch.autograd.Function):
     @staticmethod
     @torch.amp.custom_bwd(device_type="cuda")
     def backward(ctx, dlogits):
+        _first_order_only()
         x, w = ctx.saved_tensors
         dx = dw = None
         if ctx.needs_input_grad[0]:
@@ -269,6 +279,7 @@ class _MoEFFN(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dout, *unused):
+        _first_order_only()
         xp, gu, act, gates, ids, offs, pos_to_row, row_to_pos, w1b, w3b, w2b = ctx.saved_tensors
         k, E = ctx.k, ctx.E
         if dout is None:
@@ -361,6 +372,7 @@ class _MoEFFNf32(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dout, *unused):
+        _first_order_only()
         xp, g, u, act, y, gates, ids, offs, pos_to_row, row_to_pos, w1, w3, w2 = ctx.saved_tensors
         k, E = ctx.k, ctx.E
         if dout is None:
@@ -461,6 +473,7 @@ class _PreNormMoE(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dout, dlogits_ext, *unused):
+        _first_order_only()
         (x, nw, rstd, xn, wrb, xp, gu, act, gates, ids, offs, pos_to_row, row_to_pos,
          w1b, w3b, w2b) = ctx.saved_tensors
         k, E = ctx.k, ctx.E
@@ -577,6 +590,7 @@ class _ExpertsRows(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dout, *unused):
+        _first_order_only()
         xp, gu, act, offs, pos_to_row, row_to_pos, w1b, w3b, w2b = ctx.saved_tensors
         if dout is None:
             dout = torch.zeros(ctx.out_shape, dtype=ctx.x_dtype, device=xp.device)
@@ -614,6 +628,7 @@ class _ExpertsRowsF32(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dout, *unused):
+        _first_order_only()
         xp, g, u, act, offs, pos_to_row, row_to_pos, w1, w3, w2 = ctx.saved_tensors
         if dout is None:
             dout = torch.zeros(ctx.out_shape, dtype=torch.float32, device=xp.device)
